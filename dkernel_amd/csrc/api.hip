@@ -1,0 +1,185 @@
+// C-ABI entry points for the device side: argument checks (the reference's
+// Python asserts, done before any launch so that a bad shape can never reach a
+// kernel), parameter-block construction and dispatch between the MFMA kernels
+// (bf16 / fp16, head_dim 128 or 64, 64x64 blocks) and the generic kernels.
+#include <hip/hip_runtime.h>
+
+#include "common.h"
+#include "device_common.h"
+
+namespace dk {
+
+int launch_generic_fwd(const FwdParams &p, int dtype, hipStream_t stream);
+int launch_generic_bwd(const BwdParams &p, int dtype, hipStream_t stream, bool delta_only);
+bool mfma_fwd_supported(const FwdParams &p, int dtype);
+int launch_mfma_fwd(const FwdParams &p, int dtype, hipStream_t stream);
+bool mfma_bwd_supported(const BwdParams &p, int dtype);
+int launch_mfma_bwd(const BwdParams &p, int dtype, hipStream_t stream);
+bool decode_supported(const FwdParams &p, int dtype);
+size_t decode_workspace_bytes(const FwdParams &p);
+int launch_decode(const FwdParams &p, int dtype, void *workspace, size_t workspace_bytes, hipStream_t stream);
+
+static size_t elem_size(int dtype) { return dtype == DK_F32 ? 4 : 2; }
+
+static TensorView view(const dk_tensor &t) { return TensorView{t.ptr, t.stride_b, t.stride_h, t.stride_t}; }
+static RowView view(const dk_rowvec &t) { return RowView{t.ptr, t.stride_b, t.stride_h, t.stride_t}; }
+static LutView view(const dk_lut &l) {
+  return LutView{l.ptr, l.idx, l.ptr_stride_h, l.idx_stride_h, l.entry_width, l.num_heads,
+                 l.num_rows, l.block_rows, l.block_cols};
+}
+static SeqView view(const dk_seqs &s) {
+  return SeqView{s.batch, s.max_q_len, s.max_k_len, s.packed, s.q_starts, s.q_ends, s.k_starts, s.k_ends};
+}
+
+static bool vec_aligned(const dk_tensor &t, size_t es) {
+  return ((uintptr_t)t.ptr % 16 == 0) && ((t.stride_b * es) % 16 == 0) && ((t.stride_h * es) % 16 == 0) &&
+         ((t.stride_t * es) % 16 == 0);
+}
+
+static int check_lut(const dk_lut &l, const char *name, int Hq, int Hkv) {
+  DK_REQUIRE(l.ptr && l.idx, "%s look-up table is NULL", name);
+  DK_REQUIRE(l.num_heads == 1 || l.num_heads == Hkv || l.num_heads == Hq,
+             "Input (q, k) have (%d, %d) heads but the number of heads in the sparse pattern is %d", Hq, Hkv,
+             l.num_heads);
+  DK_REQUIRE(is_pow2(l.block_rows) && is_pow2(l.block_cols) && l.block_rows >= 16 && l.block_cols >= 16 &&
+                 l.block_rows <= 1024 && l.block_cols <= 1024,
+             "%s tile sizes must be powers of 2 in [16, 1024], got (%d, %d)", name, l.block_rows, l.block_cols);
+  DK_REQUIRE(l.entry_width == 1 || l.entry_width == 2, "%s entry_width must be 1 or 2", name);
+  DK_REQUIRE(l.num_rows >= 0, "%s num_rows negative", name);
+  return DK_OK;
+}
+
+static int check_common(const dk_seqs &s, int Hq, int Hkv, int D, int dtype, int causal) {
+  DK_REQUIRE(Hq >= 1 && Hkv >= 1 && Hq % Hkv == 0, "num_q_heads (%d) must be a multiple of num_kv_heads (%d)", Hq,
+             Hkv);
+  DK_REQUIRE(D >= 1 && D <= 256, "head_dim %d not in [1, 256]", D);
+  DK_REQUIRE(dtype == DK_BF16 || dtype == DK_F16 || dtype == DK_F32, "unknown dtype %d", dtype);
+  DK_REQUIRE(s.batch >= 0 && s.max_q_len >= 0 && s.max_k_len >= 0, "negative sizes");
+  DK_REQUIRE(Hq <= 65535 && s.batch <= 65535, "too many heads or sequences for one launch");
+  const bool all = s.q_starts && s.q_ends && s.k_starts && s.k_ends;
+  const bool none = !s.q_starts && !s.q_ends && !s.k_starts && !s.k_ends;
+  DK_REQUIRE(all || none, "q/k starts/ends must be given together");
+  DK_REQUIRE(!s.packed || all, "packed inputs need sequence offsets");
+  if (none && causal)
+    DK_REQUIRE(s.max_k_len >= s.max_q_len, "causal attention needs k length (%d) >= q length (%d)", s.max_k_len,
+               s.max_q_len);
+  return DK_OK;
+}
+
+static int make_fwd_params(const dk_fwd_args *a, FwdParams &p) {
+  DK_REQUIRE(a != nullptr, "args is NULL");
+  int rc = check_common(a->seqs, a->num_q_heads, a->num_kv_heads, a->head_dim, a->dtype, a->causal);
+  if (rc) return rc;
+  rc = check_lut(a->csr, "csr", a->num_q_heads, a->num_kv_heads);
+  if (rc) return rc;
+  DK_REQUIRE((int64_t)a->csr.num_rows * a->csr.block_rows >= a->seqs.max_k_len || a->seqs.packed,
+             "Input length %d is larger than the maximum length allowed (%lld)", a->seqs.max_k_len,
+             (long long)a->csr.num_rows * a->csr.block_rows);
+  const bool empty = a->seqs.batch == 0 || a->seqs.max_q_len == 0;
+  DK_REQUIRE(empty || (a->q.ptr && a->k.ptr && a->v.ptr && a->o.ptr) || a->seqs.max_k_len == 0, "q/k/v/o is NULL");
+  p.q = view(a->q);
+  p.k = view(a->k);
+  p.v = view(a->v);
+  p.o = view(a->o);
+  p.lse = view(a->lse);
+  p.csr = view(a->csr);
+  p.seqs = view(a->seqs);
+  p.Hq = a->num_q_heads;
+  p.Hkv = a->num_kv_heads;
+  p.D = a->head_dim;
+  p.causal = a->causal ? 1 : 0;
+  p.scale_log2 = a->sm_scale * kLog2e;
+  const size_t es = elem_size(a->dtype);
+  p.vec_ok = vec_aligned(a->q, es) && vec_aligned(a->k, es) && vec_aligned(a->v, es) && vec_aligned(a->o, es);
+  return DK_OK;
+}
+
+}  // namespace dk
+
+using namespace dk;
+
+extern "C" {
+
+size_t dk_fwd_workspace_bytes(const dk_fwd_args *a) {
+  FwdParams p;
+  if (make_fwd_params(a, p) != DK_OK) return 0;
+  if (a->impl != DK_IMPL_GENERIC && decode_supported(p, a->dtype)) return decode_workspace_bytes(p);
+  return 0;
+}
+
+int dk_fwd(const dk_fwd_args *a) {
+  clear_error();
+  FwdParams p;
+  int rc = make_fwd_params(a, p);
+  if (rc) return rc;
+  if (p.seqs.batch == 0 || p.seqs.max_q_len == 0) return DK_OK;
+  hipStream_t stream = (hipStream_t)a->stream;
+  if (a->impl != DK_IMPL_GENERIC) {
+    if (decode_supported(p, a->dtype) && a->workspace &&
+        a->workspace_bytes >= decode_workspace_bytes(p))
+      return launch_decode(p, a->dtype, a->workspace, a->workspace_bytes, stream);
+    if (mfma_fwd_supported(p, a->dtype)) return launch_mfma_fwd(p, a->dtype, stream);
+    if (a->impl == DK_IMPL_MFMA)
+      return fail(DK_ERR_UNSUPPORTED, "no MFMA forward kernel for dtype %d, head_dim %d, tiles (%d, %d)", a->dtype,
+                  p.D, p.csr.block_rows, p.csr.block_cols);
+  }
+  return launch_generic_fwd(p, a->dtype, stream);
+}
+
+int dk_bwd(const dk_bwd_args *a) {
+  clear_error();
+  DK_REQUIRE(a != nullptr, "args is NULL");
+  int rc = check_common(a->seqs, a->num_q_heads, a->num_kv_heads, a->head_dim, a->dtype, a->causal);
+  if (rc) return rc;
+  DK_REQUIRE(!a->seqs.q_starts && !a->seqs.packed,
+             "Currently does not support paddings or variable length inputs in backward.");
+  rc = check_lut(a->csr, "csr", a->num_q_heads, a->num_kv_heads);
+  if (rc) return rc;
+  rc = check_lut(a->csc, "csc", a->num_q_heads, a->num_kv_heads);
+  if (rc) return rc;
+  DK_REQUIRE(a->csc.entry_width == 1, "csc table cannot carry values");
+  DK_REQUIRE((int64_t)a->csr.num_rows * a->csr.block_rows >= a->seqs.max_k_len,
+             "Input length %d is larger than the maximum length allowed", a->seqs.max_k_len);
+  if (a->seqs.batch == 0 || a->seqs.max_q_len == 0) return DK_OK;
+  DK_REQUIRE(a->q.ptr && a->k.ptr && a->v.ptr && a->o.ptr && a->dout.ptr && a->dq.ptr && a->dk.ptr && a->dv.ptr,
+             "a tensor pointer is NULL");
+  DK_REQUIRE(a->lse.ptr && a->delta, "lse / delta is NULL");
+  BwdParams p;
+  p.q = view(a->q);
+  p.k = view(a->k);
+  p.v = view(a->v);
+  p.o = view(a->o);
+  p.dout = view(a->dout);
+  p.dq = view(a->dq);
+  p.dk = view(a->dk);
+  p.dv = view(a->dv);
+  p.lse = view(a->lse);
+  p.dlse = view(a->dlse);
+  p.delta = a->delta;
+  p.csr = view(a->csr);
+  p.csc = view(a->csc);
+  p.seqs = view(a->seqs);
+  p.Hq = a->num_q_heads;
+  p.Hkv = a->num_kv_heads;
+  p.D = a->head_dim;
+  p.causal = a->causal ? 1 : 0;
+  p.sm_scale = a->sm_scale;
+  p.scale_log2 = a->sm_scale * kLog2e;
+  const size_t es = elem_size(a->dtype);
+  p.vec_ok = vec_aligned(a->q, es) && vec_aligned(a->k, es) && vec_aligned(a->v, es) && vec_aligned(a->o, es) &&
+             vec_aligned(a->dout, es) && vec_aligned(a->dq, es) && vec_aligned(a->dk, es) && vec_aligned(a->dv, es);
+  hipStream_t stream = (hipStream_t)a->stream;
+  if (a->impl != DK_IMPL_GENERIC) {
+    if (mfma_bwd_supported(p, a->dtype)) {
+      rc = launch_generic_bwd(p, a->dtype, stream, /*delta_only=*/true);
+      if (rc) return rc;
+      return launch_mfma_bwd(p, a->dtype, stream);
+    }
+    if (a->impl == DK_IMPL_MFMA)
+      return fail(DK_ERR_UNSUPPORTED, "no MFMA backward kernel for dtype %d, head_dim %d, tiles (%d, %d)",
+                  a->dtype, p.D, p.csr.block_rows, p.csr.block_cols);
+  }
+  return launch_generic_bwd(p, a->dtype, stream, /*delta_only=*/false);
+}
+
+}  // extern "C"

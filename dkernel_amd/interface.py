@@ -1,0 +1,250 @@
+"""Module API: `SparseAttention`, `LocalStrideSparseAttention` and
+`combine_attn_partitions`, with the constructor / forward signatures, buffer
+names, defaults and error behaviour of the reference's dkernel/interface.py, so
+that a model written against `dkernel` runs unchanged.
+"""
+from __future__ import annotations
+
+import copy
+import math
+import warnings
+from functools import lru_cache
+from typing import Optional, Tuple
+
+import torch
+from torch import Tensor
+
+from .ops import _sparse_attention
+from .utils import (dense_to_ccol_row, get_sparse_attn_mask, is_kv_cache_efficient,
+                    merge_split_fwd_kernel_blocks, multiple_of, verify_sparse_pattern, zero_stride)
+
+
+class SparseAttention(torch.nn.Module):
+    """Block-sparse attention over a user-given block pattern.
+
+    Arguments
+    =========
+    block_size: sparse block size, a power of 2, at least 16.
+    sparse_pattern: 2-D or 3-D (per head) bool / uint8 tensor, 1 = attend.
+    causal: default True.
+    seq_dim: None / 1 -> (batch, seq, heads, dim); 2 -> (batch, heads, seq, dim).
+        Ignored for packed variable-length (3-D) inputs.
+    block_m, block_n: kernel tile sizes on q and k (powers of 2, >= 16).
+        Default block_m = max(block_size, 64) if causal else block_size,
+        block_n = block_size.
+    kwargs: "out" (output tensor), "d_splits" (accepted, unused), "inference"
+        (skip saving the log-sum-exp for backward; default: no input needs grad).
+
+    forward(q, k, v, sm_scale=None, *, cu_seqlen_k, cu_seqlen_q, left_paddings,
+            seqlens, return_lse, split_qkv): see the method.
+
+    Reference: dkernel/interface.py:18-215.
+    """
+
+    def __init__(self,
+                 block_size: int,
+                 sparse_pattern: Tensor,
+                 *,
+                 causal: bool = True,
+                 seq_dim: Optional[int] = None,
+                 block_m: Optional[int] = None,
+                 block_n: Optional[int] = None,
+                 **kwargs):
+        super().__init__()
+
+        def _check_block_size(block_size: int, name: str):
+            if block_size is not None:
+                assert block_size >= 16 and math.log2(block_size) % 1 == 0, \
+                    f"{name} must be power of 2 and at least 16, but {block_size} is given."
+
+        _check_block_size(block_size, "block_size")
+        _check_block_size(block_m, "block_m")
+        _check_block_size(block_n, "block_n")
+
+        if block_m is None:
+            block_m = max(block_size, 64) if causal else block_size
+        if block_n is None:
+            block_n = block_size
+
+        sparse_pattern = sparse_pattern.to(torch.uint8)
+        if sparse_pattern.dim() == 2:
+            sparse_pattern = zero_stride(sparse_pattern[None])
+        verify_sparse_pattern(sparse_pattern)
+        if causal and not is_kv_cache_efficient(sparse_pattern, block_size, block_size):
+            warnings.warn("The provided sparse_pattern is not efficient for KV cache, "
+                          "i.e., KV cache needed for later tokens are not used in "
+                          "earlier tokens. This may result in unexpected larger KV cache.")
+
+        self.block_size = block_size
+        self.block_m = block_m
+        self.block_n = block_n
+        self.seq_dim = seq_dim
+        self.max_seqlen = max(sparse_pattern.shape[1:]) * block_size
+        self.kwargs = copy.copy(kwargs)
+        self.kwargs["max_seqlen"] = self.max_seqlen
+        self.kwargs['causal'] = causal
+
+        if not causal:
+            # merged q tiles are a causal-only optimisation
+            assert self.block_m <= block_size
+            assert self.block_n <= block_size
+
+        layout_csr = list(merge_split_fwd_kernel_blocks(block_size, sparse_pattern,
+                                                        self.block_m, self.block_n, causal=causal))
+        # the dK/dV pass always walks columns at the sparse block size
+        self.block_m2, self.block_n2 = self.block_size, self.block_size
+        layout_csc = list(dense_to_ccol_row(sparse_pattern, include_values=False))
+
+        if layout_csr[0].dim() == 1:
+            layout_csr = [x[None] for x in layout_csr]
+            layout_csc = [x[None] for x in layout_csc]
+        if layout_csr[0].size(0) == 1:
+            layout_csr = [zero_stride(x) for x in layout_csr]
+            layout_csc = [zero_stride(x) for x in layout_csc]
+
+        self.register_buffer("layout_csr_crow", layout_csr[0].to(torch.int32), persistent=False)
+        self.register_buffer("layout_csr_col", layout_csr[1].to(torch.int32), persistent=False)
+        self.register_buffer("layout_csc_ccol", layout_csc[0].to(torch.int32), persistent=False)
+        self.register_buffer("layout_csc_row", layout_csc[1].to(torch.int32), persistent=False)
+
+    def forward(self,
+                q: Tensor,
+                k: Optional[Tensor] = None,
+                v: Optional[Tensor] = None,
+                sm_scale: Optional[float] = None,
+                *,
+                cu_seqlen_k: Optional[Tensor] = None,
+                cu_seqlen_q: Optional[Tensor] = None,
+                left_paddings: Optional[Tensor] = None,
+                seqlens: Optional[Tensor] = None,
+                return_lse: bool = False,
+                split_qkv: Optional[callable] = None):
+        """
+        q, k, v:
+            packing: with k and v None, `q` holds qkv and `split_qkv(q)` gives
+            (q, k, v); with only v None, `k` holds kv and `split_qkv(k)` gives (k, v).
+            shapes: (batch, seq, heads, dim) [seq_dim 1 / None] or
+            (batch, heads, seq, dim) [seq_dim 2]; for inference also 4-D with
+            `left_paddings` / `seqlens`, or packed 3-D (total_tokens, heads, dim)
+            with `cu_seqlen_k` (and `cu_seqlen_q`).
+        sm_scale: softmax scale, default 1 / sqrt(dim).
+        return_lse: also return the natural-log softmax normaliser, (batch,
+            heads, seq) for 4-D inputs and (heads, total_tokens) for packed ones.
+        """
+        inf_kwargs = {"cu_seqlen_k": cu_seqlen_k,
+                      "cu_seqlen_q": cu_seqlen_q,
+                      "left_paddings": left_paddings,
+                      "seqlens": seqlens}
+        kwargs = copy.copy(self.kwargs)
+        kwargs["return_lse"] = return_lse
+        kwargs['split_qkv'] = split_qkv
+        output, lse = _sparse_attention.apply(
+            q, k, v, sm_scale,
+            (self.layout_csr_crow, self.layout_csr_col, self.block_m, self.block_n),
+            (self.layout_csc_ccol, self.layout_csc_row, self.block_m2, self.block_n2),
+            self.seq_dim, inf_kwargs, kwargs)
+        if return_lse:
+            return output, lse
+        return output
+
+
+@lru_cache(maxsize=8)
+class LocalStrideSparseAttention(SparseAttention):
+    """Local window + vertical stride pattern with per-head shifted columns
+    (the Phi-3-small pattern).  As in the reference the class is wrapped in
+    `functools.lru_cache(maxsize=8)`: identical constructor arguments return the
+    same cached module.
+
+    num_heads: number of q heads.
+    max_seq_len: longest sequence the module will see (rounded up to a multiple
+        of max(block_size, block_m, block_n, 64)).
+    block_size / local_blocks / vert_stride: sparse block size, number of local
+        blocks (including the diagonal one), and 1-in-`vert_stride` vertical columns.
+    homo_head: one pattern for every head.
+    num_dense_heads: the last `num_dense_heads` kv heads attend densely.
+    num_kv_heads: grouped-query attention; q heads of a group share a pattern.
+    active_head_range: (start, end) q heads handled by this rank (head /
+        tensor parallelism).
+    head_sliding_offset: shifts which head owns vertical column 0.
+
+    Reference: dkernel/interface.py:218-300.
+    """
+
+    def __init__(self,
+                 num_heads: int,
+                 max_seq_len: int,
+                 block_size: int,
+                 local_blocks: int,
+                 vert_stride: int,
+                 *,
+                 homo_head: bool = False,
+                 num_dense_heads: int = 0,
+                 num_kv_heads: Optional[int] = None,
+                 active_head_range: Optional[Tuple[int, int]] = None,
+                 head_sliding_offset: int = 0,
+                 block_m: Optional[int] = None,
+                 block_n: Optional[int] = None,
+                 causal: bool = True,
+                 **kwargs):
+        assert vert_stride >= 1, "Vertical stride should be position integer. Value 1 will collapse to dense attention."
+        if vert_stride > 1:
+            assert local_blocks >= 1, "Token in the first block will attend to nothing in some blocks."
+        self.max_seq_len = multiple_of(max_seq_len, max([block_size, block_m or 1, block_n or 1, 64]))
+        self.num_heads = num_heads
+        self.num_kv_heads = num_kv_heads
+        self.local_blocks = local_blocks
+        self.vert_stride = vert_stride
+        self.homo_head = homo_head
+        self.num_dense_heads = num_dense_heads
+        sparse_pattern = get_sparse_attn_mask(num_heads, self.max_seq_len,
+                                              block_size=block_size,
+                                              local_blocks=local_blocks,
+                                              vert_stride=vert_stride,
+                                              homo_head=homo_head,
+                                              dtype=torch.uint8,
+                                              num_kv_heads=num_kv_heads,
+                                              head_sliding_offset=head_sliding_offset,
+                                              num_dense_heads=num_dense_heads,
+                                              causal=causal)[1]
+        # homogeneous heads share one pattern, nothing to slice
+        if (not homo_head) and (active_head_range is not None) and sparse_pattern.size(0) > 1:
+            assert isinstance(active_head_range, tuple)
+            assert len(active_head_range) == 2, '"active_head_range" should be a tuple of start/end index of the heads.'
+            h_start, h_end = active_head_range
+            sparse_pattern = sparse_pattern[h_start:h_end]
+        super().__init__(block_size, sparse_pattern, block_m=block_m, block_n=block_n, causal=causal, **kwargs)
+
+
+def combine_attn_partitions(*x: Tuple[Tensor, Tensor], hdim=1):
+    """Merge attention results computed over disjoint K/V partitions:
+    out = sum_p softmax_p(lse_p) * out_p.  Each argument is (out_p, lse_p).
+
+    `hdim` is the head dimension of the outputs: with the default 1 the
+    outputs are (batch, heads, seq, dim) and line up with the (batch, heads,
+    seq) log-sum-exps as in the reference (dkernel/interface.py:303-324); when
+    the head dimension comes right before `dim` -- (batch, seq, heads, dim) with
+    hdim=2, or packed (tokens, heads, dim) -- the (.., heads, seq) log-sum-exps
+    are transposed to match.  Partitions in which a row saw no key (lse = -inf)
+    get weight 0.
+    """
+    assert len(x) >= 2 and len(x[0]) == 2
+    outputs, weights = list(zip(*x))
+    weights = torch.stack(weights, dim=0)
+    outputs = torch.stack(outputs, dim=0)
+    head_before_dim = (hdim % (outputs.dim() - 1)) == outputs.dim() - 3
+    mismatch = weights.shape[1:] != outputs.shape[1:-1]
+    if (head_before_dim and weights.dim() >= 3 and
+            weights.transpose(-1, -2).shape[1:] == outputs.shape[1:-1]) or \
+            (mismatch and weights.transpose(-1, -2).shape[1:] == outputs.shape[1:-1]):
+        weights = weights.transpose(-1, -2)
+    weights = weights.softmax(dim=0)
+    weights = torch.where(torch.isnan(weights), torch.zeros_like(weights), weights)
+    output = (outputs * weights.unsqueeze(-1)).sum(0).type_as(outputs)
+    return output
+
+
+__all__ = [
+    "SparseAttention",
+    "LocalStrideSparseAttention",
+    "combine_attn_partitions",
+]

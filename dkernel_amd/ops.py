@@ -1,0 +1,412 @@
+"""autograd Function and host launchers, mirroring the reference's
+dkernel/ops/__init__.py (dispatch, packing, error behaviour) and the host
+halves of sparse_attn_fwd.py / sparse_attn_bwd.py / sparse_attn_inference.py.
+The device work goes through the C ABI of libdkernel_hip.so; there is no
+other execution path (CPU tensors are refused).
+
+Differences from the reference, all supersets: grouped-query attention works
+on every path (kv head = q head // group), LSE is returned whenever asked
+(also from padded and packed inputs, and without grad), and no launcher
+synchronises with the host.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import math
+from typing import Dict, Optional, Tuple, Union
+
+import torch
+from torch import Tensor
+
+from . import _lib
+
+_DTYPES = {torch.bfloat16: _lib.DK_BF16, torch.float16: _lib.DK_F16, torch.float32: _lib.DK_F32}
+
+# Kernel selection for tests and benchmarks: "auto", "generic" or "mfma".
+_IMPL = {"auto": _lib.DK_IMPL_AUTO, "generic": _lib.DK_IMPL_GENERIC, "mfma": _lib.DK_IMPL_MFMA}
+_impl = _lib.DK_IMPL_AUTO
+
+
+def set_impl(name: str) -> None:
+    global _impl
+    _impl = _IMPL[name]
+
+
+def _require_gpu(*xs: Tensor) -> None:
+    for x in xs:
+        if not x.is_cuda:
+            raise RuntimeError(
+                "dkernel_amd runs on ROCm (MI355X) tensors only; got a tensor on "
+                f"{x.device}. There is no CPU execution path.")
+    if xs[0].dtype not in _DTYPES:
+        raise TypeError(f"unsupported dtype {xs[0].dtype}; use bfloat16, float16 or float32")
+    assert all(x.dtype == xs[0].dtype for x in xs), "q, k, v must share a dtype"
+
+
+def _unit_last(x: Tensor) -> Tensor:
+    return x if x.stride(-1) == 1 else x.contiguous()
+
+
+def _tensor4(x: Tensor, hdim: int, seq_dim: int) -> _lib.Tensor:
+    return _lib.Tensor(x.data_ptr(), x.stride(0), x.stride(hdim), x.stride(seq_dim))
+
+
+def _tensor3(x: Tensor) -> _lib.Tensor:  # packed (tokens, heads, dim)
+    return _lib.Tensor(x.data_ptr(), 0, x.stride(1), x.stride(0))
+
+
+def _rowvec(x: Optional[Tensor], strides=None) -> _lib.RowVec:
+    if x is None:
+        return _lib.RowVec(None, 0, 0, 0)
+    sb, sh, st = strides if strides is not None else x.stride()
+    return _lib.RowVec(x.data_ptr(), sb, sh, st)
+
+
+def _lut(layout: Tuple[Tensor, Tensor, int, int], device) -> _lib.Lut:
+    ptr, idx, block_rows, block_cols = layout
+    assert ptr.dtype == torch.int32 and idx.dtype == torch.int32
+    assert ptr.device == device and idx.device == device, \
+        "sparse layout is on another device than q; move the module with .to(device)"
+    if ptr.dim() == 1:
+        ptr, idx = ptr[None], idx[None]
+    assert ptr.stride(-1) == 1
+    width = 1
+    if idx.dim() == 3:
+        assert idx.size(2) == 2 and idx.stride(2) == 1 and idx.stride(1) == 2
+        width = 2
+    else:
+        assert idx.stride(-1) == 1 or idx.size(-1) <= 1
+    return _lib.Lut(ptr.data_ptr(), idx.data_ptr(), ptr.stride(0), idx.stride(0), width,
+                    ptr.size(0), ptr.size(1) - 1, int(block_rows), int(block_cols))
+
+
+def _stream() -> C.c_void_p:
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _run_fwd(args: _lib.FwdArgs, device) -> None:
+    lib = _lib.lib()
+    need = lib.dk_fwd_workspace_bytes(C.byref(args))
+    ws = None
+    if need:
+        ws = torch.empty(need, dtype=torch.uint8, device=device)
+        args.workspace, args.workspace_bytes = ws.data_ptr(), need
+    _lib.check(lib.dk_fwd(C.byref(args)))
+
+
+def _forward(ctx, q: Tensor, k: Tensor, v: Tensor, sm_scale: float,
+             layout_csr: Tuple[Tensor, Tensor, int, int],
+             seq_dim: int = 1,
+             inference: Optional[bool] = None,
+             out: Optional[Tensor] = None,
+             d_splits: Optional[int] = None,
+             max_seqlen: Optional[int] = None,
+             return_lse: bool = False,
+             causal=True,
+             split_qkv=None) -> Tuple[Tensor, Optional[Tensor]]:
+    """Unpadded 4-D forward (training, prefill, single-token decode).
+    Reference: dkernel/ops/sparse_attn_fwd.py:383-567.  `d_splits` is accepted
+    and ignored (a Triton shared-memory workaround)."""
+    assert seq_dim in [2, 1]
+    hdim = 3 - seq_dim
+    assert q.shape[-1] == k.shape[-1] == v.shape[-1]
+    assert k.shape[seq_dim] == v.shape[seq_dim]
+    qlen, klen = q.size(seq_dim), k.size(seq_dim)
+    num_heads, num_kv_heads = q.size(hdim), k.size(hdim)
+    if max_seqlen is not None:
+        assert klen <= max_seqlen
+    num_head_patterns = layout_csr[0].size(0) if layout_csr[0].dim() == 2 else 1
+    if num_head_patterns > 1:
+        assert num_head_patterns in [num_heads, num_kv_heads]
+
+    q, k, v = _unit_last(q), _unit_last(k), _unit_last(v)
+    o = out if out is not None else q.new_empty(q.shape).contiguous()
+    if inference is None:
+        inference = (not q.requires_grad) and (not k.requires_grad) and (not v.requires_grad)
+    need_lse = return_lse or not inference
+    lse = torch.empty((q.size(0), num_heads, qlen), dtype=torch.float32, device=q.device) if need_lse else None
+
+    args = _lib.FwdArgs()
+    args.q, args.k, args.v, args.o = (_tensor4(x, hdim, seq_dim) for x in (q, k, v, o))
+    args.lse = _rowvec(lse)
+    args.csr = _lut(layout_csr, q.device)
+    args.seqs = _lib.Seqs(q.size(0), qlen, klen, 0, None, None, None, None)
+    args.num_q_heads, args.num_kv_heads, args.head_dim = num_heads, num_kv_heads, q.size(-1)
+    args.dtype, args.causal, args.impl = _DTYPES[q.dtype], int(bool(causal)), _impl
+    args.sm_scale = float(sm_scale)
+    args.stream = _stream()
+    _run_fwd(args, q.device)
+
+    ctx.save_for_backward(q, k, v, o, lse)
+    ctx.sm_scale = sm_scale
+    ctx.seq_dim = seq_dim
+    ctx.hdim = hdim
+    ctx.causal = causal
+    return o, (lse if return_lse else None)
+
+
+def _backward(ctx, do: Tensor, dlse: Optional[Tensor],
+              dq: Optional[Tensor] = None, dk: Optional[Tensor] = None, dv: Optional[Tensor] = None
+              ) -> Tuple[Tensor, Tensor, Tensor]:
+    """dQ, dK, dV.  Reference: dkernel/ops/sparse_attn_bwd.py:724-852."""
+    q, k, v, o, lse = ctx.saved_tensors
+    hdim, seq_dim = ctx.hdim, ctx.seq_dim
+    assert lse is not None, "forward ran in inference mode; backward needs the saved log-sum-exp"
+    do = _unit_last(do)
+
+    def _check_or_new(x, like):
+        if x is not None:
+            assert x.shape == like.shape
+            assert x.stride(-1) == 1
+            return x
+        return like.new_empty(like.shape)
+
+    dq, dk, dv = _check_or_new(dq, q), _check_or_new(dk, k), _check_or_new(dv, v)
+    B, Hq, Lq = q.size(0), q.size(hdim), q.size(seq_dim)
+    delta = torch.empty((B, Hq, Lq), dtype=torch.float32, device=q.device)
+
+    args = _lib.BwdArgs()
+    for name, x in (("q", q), ("k", k), ("v", v), ("o", o), ("dout", do), ("dq", dq), ("dk", dk), ("dv", dv)):
+        setattr(args, name, _tensor4(x, hdim, seq_dim))
+    args.lse = _rowvec(lse)
+    if dlse is not None:
+        assert dlse.shape == lse.shape
+        args.dlse = _rowvec(dlse.float() if dlse.dtype != torch.float32 else dlse)
+    else:
+        args.dlse = _rowvec(None)
+    args.delta = delta.data_ptr()
+    args.csr = _lut(ctx.layout_csr, q.device)
+    args.csc = _lut(ctx.layout_csc, q.device)
+    args.seqs = _lib.Seqs(B, Lq, k.size(seq_dim), 0, None, None, None, None)
+    args.num_q_heads, args.num_kv_heads, args.head_dim = Hq, k.size(hdim), q.size(-1)
+    args.dtype, args.causal, args.impl = _DTYPES[q.dtype], int(bool(ctx.causal)), _impl
+    args.sm_scale = float(ctx.sm_scale)
+    args.stream = _stream()
+    _lib.check(_lib.lib().dk_bwd(C.byref(args)))
+    return dq, dk, dv
+
+
+def padded_sparse_attn(q: Tensor, k: Tensor, v: Tensor, sm_scale: float,
+                       sparse_layout: Tuple[Tensor, Tensor, int, int], *,
+                       left_paddings: Optional[Tensor] = None,
+                       seqlens: Optional[Tensor] = None,
+                       max_seqlen: Optional[int] = None,
+                       seq_dim: int = 1,
+                       d_splits: Optional[int] = None,
+                       out: Optional[Tensor] = None,
+                       inference: bool = True,
+                       causal: bool = True,
+                       return_lse: bool = False):
+    """4-D inputs with left paddings and / or explicit sequence lengths; q has
+    either one token per sequence (decode) or the same padded length as k.
+    Reference: dkernel/ops/sparse_attn_inference.py:10-147.  Padding rows of
+    the output are zero.  Nothing here reads device memory on the host."""
+    assert seq_dim in (1, 2)
+    hdim = 3 - seq_dim
+    batches, head_size = q.size(0), q.size(3)
+    q_len, k_len = q.size(seq_dim), k.size(seq_dim)
+    num_heads, num_kv_heads = q.size(hdim), k.size(hdim)
+    assert q.dim() == k.dim() == v.dim() == 4
+    assert num_heads % num_kv_heads == 0
+    assert q.size(0) == k.size(0) and q.size(3) == k.size(3)
+    assert k.shape == v.shape
+    assert q_len == 1 or q_len == k_len, \
+        (f'q length can only 1 for decoding or the same as k length for prefilling, '
+         f'but got {q_len=}, {k_len=}.')
+    if max_seqlen:
+        assert k_len <= max_seqlen, \
+            f'k has seqlen {k_len} while max sequence length is set to {max_seqlen}.'
+    q, k, v = _unit_last(q), _unit_last(k), _unit_last(v)
+    out = out if out is not None else q.new_zeros(q.shape)
+
+    dev = q.device
+    if left_paddings is not None:
+        assert left_paddings.shape == (batches,)
+        k_starts = left_paddings.to(dev, dtype=torch.int32).contiguous()
+    else:
+        k_starts = torch.zeros((batches,), dtype=torch.int32, device=dev)
+    if seqlens is not None:
+        # ends beyond the padded length are clamped on the device
+        k_ends = k_starts + seqlens.to(dev, dtype=torch.int32)
+    else:
+        k_ends = torch.full_like(k_starts, k_len)
+    if q_len == 1:
+        q_starts = torch.zeros_like(k_starts)
+        q_ends = q_starts + 1
+    else:
+        q_starts, q_ends = k_starts, k_ends
+
+    lse = None
+    if return_lse:
+        lse = torch.full((batches, num_heads, q_len), float("-inf"), dtype=torch.float32, device=dev)
+    args = _lib.FwdArgs()
+    args.q, args.k, args.v, args.o = (_tensor4(x, hdim, seq_dim) for x in (q, k, v, out))
+    args.lse = _rowvec(lse)
+    args.csr = _lut(sparse_layout, dev)
+    args.seqs = _lib.Seqs(batches, q_len, k_len, 0, q_starts.data_ptr(), q_ends.data_ptr(),
+                          k_starts.data_ptr(), k_ends.data_ptr())
+    args.num_q_heads, args.num_kv_heads, args.head_dim = num_heads, num_kv_heads, head_size
+    args.dtype, args.causal, args.impl = _DTYPES[q.dtype], int(bool(causal)), _impl
+    args.sm_scale = float(sm_scale)
+    args.stream = _stream()
+    _run_fwd(args, dev)
+    return (out, lse) if return_lse else out
+
+
+def varlen_sparse_attn(q: Tensor, k: Tensor, v: Tensor,
+                       cu_seqlens_k: Tensor, cu_seqlens_q: Optional[Tensor],
+                       sm_scale: float,
+                       sparse_layout: Tuple[Tensor, Tensor, int, int], *,
+                       max_seqlen: int = None,
+                       d_splits: Optional[int] = None,
+                       out: Optional[Tensor] = None,
+                       inference: bool = True,
+                       causal: bool = True,
+                       return_lse: bool = False):
+    """Packed variable-length inputs (total_tokens, heads, head_dim) with
+    cumulative sequence lengths.  Reference:
+    dkernel/ops/sparse_attn_inference.py:150-287.  The query tokens of a
+    sequence are the last q_len positions of its keys (q_len == k_len for
+    prefill, 1 for decode; anything between is chunked prefill).  LSE, when
+    asked for, has shape (heads, total_q_tokens)."""
+    assert isinstance(sparse_layout, (list, tuple))
+    _, num_heads, head_size = q.shape
+    batch_size = cu_seqlens_k.size(0) - 1
+    assert q.dim() == k.dim() == v.dim() == 3
+    assert q.size(1) % k.size(1) == 0
+    assert q.size(2) == k.size(2)
+    assert k.shape == v.shape
+    assert cu_seqlens_k.dim() == 1
+    dev = q.device
+    if cu_seqlens_q is None:
+        if q.size(0) == batch_size:  # decoding only
+            cu_seqlens_q = torch.arange(0, batch_size + 1, dtype=torch.int32, device=dev)
+        elif q.size(0) == k.size(0):
+            cu_seqlens_q = cu_seqlens_k
+        else:
+            raise ValueError("cu_seqlens_q must be specified if it mix of prefilling and decoding.")
+    else:
+        assert cu_seqlens_k.size(0) == cu_seqlens_q.size(0)
+    cu_q = cu_seqlens_q.to(dev, dtype=torch.int32).contiguous()
+    cu_k = cu_seqlens_k.to(dev, dtype=torch.int32).contiguous()
+    q, k, v = _unit_last(q), _unit_last(k), _unit_last(v)
+    out = out if out is not None else q.new_empty(q.shape)
+    lse = torch.full((num_heads, q.size(0)), float("-inf"), dtype=torch.float32, device=dev) if return_lse else None
+
+    args = _lib.FwdArgs()
+    args.q, args.k, args.v, args.o = (_tensor3(x) for x in (q, k, v, out))
+    args.lse = _rowvec(lse, (0, lse.stride(0), lse.stride(1))) if lse is not None else _rowvec(None)
+    args.csr = _lut(sparse_layout, dev)
+    isz = cu_q.element_size()
+    args.seqs = _lib.Seqs(batch_size, q.size(0), k.size(0), 1,
+                          cu_q.data_ptr(), cu_q.data_ptr() + isz, cu_k.data_ptr(), cu_k.data_ptr() + isz)
+    args.num_q_heads, args.num_kv_heads, args.head_dim = num_heads, k.size(1), head_size
+    args.dtype, args.causal, args.impl = _DTYPES[q.dtype], int(bool(causal)), _impl
+    args.sm_scale = float(sm_scale)
+    args.stream = _stream()
+    _run_fwd(args, dev)
+    return (out, lse) if return_lse else out
+
+
+def get_qkv_and_pack_mode(q: Tensor, k: Optional[Tensor], v: Optional[Tensor], split_qkv=None):
+    """Unpack `qkv` (k, v None) or `kv` (v None) with the user's callable.
+    Reference: dkernel/ops/__init__.py:128-149."""
+    qkv_pack_mode = 'split_qkv'
+    packed_shape = None
+    if v is None:
+        assert split_qkv is not None, "Callable `split_qkv` must be specified if qkv or kv are packed."
+        if k is None:
+            packed_shape = q.shape
+            q, k, v = split_qkv(q)
+            qkv_pack_mode = 'packed_qkv'
+        else:
+            packed_shape = k.shape
+            k, v = split_qkv(k)
+            qkv_pack_mode = 'packed_kv'
+    return (q, k, v), (packed_shape, qkv_pack_mode, split_qkv)
+
+
+class _sparse_attention(torch.autograd.Function):
+    """Same 9-argument form and dispatch as the reference's
+    dkernel/ops/__init__.py:10-125."""
+
+    @staticmethod
+    def forward(ctx, q: Tensor, k: Optional[Tensor], v: Optional[Tensor], sm_scale: float,
+                layout_csr: Tuple[Tensor, Tensor, int, int],
+                layout_csc: Tuple[Tensor, Tensor, int, int],
+                seq_dim: Optional[int], inf_kwargs: Dict, kwargs: Dict):
+        (q, k, v), (packed_shape, packed_mode, split_qkv) = \
+            get_qkv_and_pack_mode(q, k, v, split_qkv=kwargs.get("split_qkv", None))
+        _require_gpu(q, k, v)
+        ctx.layout_csr = layout_csr
+        ctx.layout_csc = layout_csc
+        ctx.packed_shape = packed_shape
+        ctx.packed_mode = packed_mode
+        ctx.split_qkv = split_qkv
+
+        seq_dim = 1 if seq_dim is None else seq_dim
+        max_seqlen = kwargs.get("max_seqlen", None)
+        causal = kwargs.get("causal", True)
+        return_lse = kwargs.get("return_lse", False)
+        lse = None
+
+        assert q.dim() in (3, 4)
+        hdim = 3 - (seq_dim or 1) if q.dim() == 4 else 1
+        layout_csr_crow = layout_csr[0]
+        assert layout_csr_crow.size(0) in [1, k.size(hdim), q.size(hdim)], \
+            (f"Input (q, k) have ({q.size(hdim)}, {k.size(hdim)}) heads"
+             f"but the number of heads in the sparse pattern is {layout_csr_crow.size(0)}")
+        sm_scale = sm_scale or 1. / math.sqrt(float(q.size(-1)))
+
+        if q.dim() == 3:
+            assert inf_kwargs.get("cu_seqlen_k", None) is not None
+            ctx.support_backward = False
+            ctx.message = "Currently does not suppoort variable length inputs. WIP."
+            res = varlen_sparse_attn(q, k, v, inf_kwargs["cu_seqlen_k"], inf_kwargs.get("cu_seqlen_q", None),
+                                     sm_scale, layout_csr, max_seqlen=max_seqlen, causal=causal,
+                                     return_lse=return_lse)
+            output, lse = res if return_lse else (res, None)
+        else:
+            assert k.size(seq_dim) <= max_seqlen, \
+                (f"Input length {k.size(seq_dim)} is larger "
+                 f"than the maximum length allowed ({max_seqlen})")
+            left_paddings = inf_kwargs.get("left_paddings", None)
+            seqlens = inf_kwargs.get("seqlens", None)
+            if (left_paddings is not None) or (seqlens is not None):
+                ctx.support_backward = False
+                ctx.message = "Currently does not support paddings in inputs. WIP."
+                res = padded_sparse_attn(q, k, v, sm_scale, layout_csr, left_paddings=left_paddings,
+                                         seqlens=seqlens, seq_dim=seq_dim, max_seqlen=max_seqlen,
+                                         causal=causal, return_lse=return_lse)
+                output, lse = res if return_lse else (res, None)
+            else:
+                ctx.support_backward = True
+                ctx.message = ""
+                fwd_kwargs = {k_: v_ for k_, v_ in kwargs.items()
+                              if k_ in ("inference", "out", "d_splits", "max_seqlen", "return_lse",
+                                        "causal", "split_qkv")}
+                output, lse = _forward(ctx, q, k, v, sm_scale, layout_csr, seq_dim=seq_dim, **fwd_kwargs)
+        return output, lse
+
+    @staticmethod
+    def backward(ctx, do: Tensor, dlse: Optional[Tensor]) -> Tuple[Union[Tensor, None], ...]:
+        assert ctx.support_backward, ctx.message
+        q, k = ctx.saved_tensors[:2]
+        dq, dk, dv = None, None, None
+        if ctx.packed_mode == 'packed_qkv':
+            dqkv = q.new_empty(ctx.packed_shape)
+            dq, dk, dv = ctx.split_qkv(dqkv)
+        elif ctx.packed_mode == 'packed_kv':
+            dkv = k.new_empty(ctx.packed_shape)
+            dk, dv = ctx.split_qkv(dkv)
+        dq, dk, dv = _backward(ctx, do, dlse, dq=dq, dk=dk, dv=dv)[:3]
+        if ctx.packed_mode == 'packed_qkv':
+            grads = (dqkv, None, None)
+        elif ctx.packed_mode == 'packed_kv':
+            grads = (dq, dkv, None)
+        else:
+            grads = (dq, dk, dv)
+        return grads + (None,) * 6
+
+
+__all__ = ["_sparse_attention", "padded_sparse_attn", "varlen_sparse_attn", "get_qkv_and_pack_mode", "set_impl"]

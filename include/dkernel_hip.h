@@ -1,0 +1,176 @@
+/*
+ * dkernel_hip.h -- C ABI of libdkernel_hip.so, the gfx950 (MI355X) block-sparse
+ * attention engine.  Plain pointers, sizes and element strides only; the
+ * library never allocates, frees or keeps caller memory, never synchronises
+ * the device, and launches on the hipStream_t handed in.
+ *
+ * Every function returns 0 (DK_OK) or a negative code; dk_last_error() gives
+ * the message of the calling thread's last failure.
+ *
+ * Each entry point names the interface of the reference (linxihui/dkernel)
+ * that it replaces.
+ */
+#ifndef DKERNEL_HIP_H
+#define DKERNEL_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DK_OK 0
+#define DK_ERR_INVALID (-1)     /* argument check failed (the reference's Python asserts) */
+#define DK_ERR_UNSUPPORTED (-2) /* shape / dtype without a kernel */
+#define DK_ERR_HIP (-3)         /* a HIP runtime call failed */
+
+enum dk_dtype { DK_BF16 = 0, DK_F16 = 1, DK_F32 = 2 };
+enum dk_impl { DK_IMPL_AUTO = 0, DK_IMPL_GENERIC = 1, DK_IMPL_MFMA = 2 };
+
+int dk_version(void);              /* 10000*major + 100*minor + patch */
+const char *dk_last_error(void);   /* thread-local, never NULL */
+
+/* --------------------------------------------------------------------------
+ * Host side: layout / look-up-table builder (runs on the CPU, no GPU needed)
+ * -------------------------------------------------------------------------- */
+
+/* Block mask of the local + vertical-stride pattern, out[num_heads][nb_q][nb_k]
+ * (uint8, 1 = attend).  Replaces the mask arithmetic of get_sparse_attn_mask,
+ * dkernel/utils.py:157-215.  num_heads is the number of pattern heads (1 for
+ * homo_head); kv head of pattern head h is h / (num_heads / num_kv_heads);
+ * the LAST num_dense_heads kv heads are dense.  relative != 0 selects the
+ * 'relative' vertical positions of utils.py:197-211. */
+int dk_local_stride_mask(int32_t num_heads, int32_t num_kv_heads, int32_t nb_q, int32_t nb_k,
+                         int32_t local_left, int32_t local_right, int32_t vert_stride,
+                         int32_t num_dense_heads, int32_t head_sliding_step,
+                         int32_t head_sliding_offset, int32_t q_start_block,
+                         int32_t kv_start_block, int32_t causal, int32_t relative, uint8_t *out);
+
+/* CSR of an int32 pattern[H][M][N] given by element strides (pass the strides
+ * of the transpose for CSC).  Pass 1 fills ptr[H][M+1] and *max_nnz; pass 2
+ * fills idx[H][width] (right-padded with -1) and, if val != NULL,
+ * val[H][width] (padded with 0).  Replaces to_csr / dense_to_crow_col /
+ * dense_to_ccol_row, dkernel/utils.py:19-24, :27-65, :91-95. */
+int dk_csr_count(const int32_t *pattern, int32_t H, int32_t M, int32_t N, int64_t stride_h,
+                 int64_t stride_m, int64_t stride_n, int32_t *ptr, int32_t *max_nnz);
+int dk_csr_fill(const int32_t *pattern, int32_t H, int32_t M, int32_t N, int64_t stride_h,
+                int64_t stride_m, int64_t stride_n, int32_t width, int32_t *idx, int32_t *val);
+
+/* Pattern at kernel-tile granularity (split to block_m x block_n sub-blocks,
+ * sub-blocks wholly above the token diagonal dropped when prune_above_diagonal,
+ * then groups of block_m / block_size row blocks merged with value
+ * micro_M = (last non-empty sub-row + 1) * block_size).  Replaces the dense
+ * stage of merge_split_fwd_kernel_blocks, dkernel/utils.py:286-307.
+ * dk_tile_pattern_shape gives the output shape and whether values (merged
+ * rows) are meaningful. */
+int dk_tile_pattern_shape(int32_t M, int32_t N, int32_t block_size, int32_t block_m,
+                          int32_t block_n, int32_t *out_m, int32_t *out_n, int32_t *merged);
+int dk_tile_pattern(const uint8_t *pattern, int32_t H, int32_t M, int32_t N, int32_t block_size,
+                    int32_t block_m, int32_t block_n, int32_t prune_above_diagonal,
+                    int32_t *out /* [H][out_m][out_n] */);
+
+/* 1 if the pattern is KV-cache friendly, 0 if not, <0 on error.  Replaces
+ * is_kv_cache_efficient, dkernel/utils.py:232-245. */
+int dk_kv_cache_efficient(const uint8_t *pattern, int32_t H, int32_t M, int32_t N,
+                          int32_t block_m, int32_t block_n);
+
+/* --------------------------------------------------------------------------
+ * Device side
+ * -------------------------------------------------------------------------- */
+
+/* A (batch, head, token, dim) view: element strides for batch / head / token,
+ * dim stride must be 1.  Packed variable-length tensors use stride_b = 0. */
+typedef struct dk_tensor {
+  void *ptr;
+  int64_t stride_b, stride_h, stride_t;
+} dk_tensor;
+
+/* A per-row fp32 quantity (LSE, dLSE): element strides batch / head / token. */
+typedef struct dk_rowvec {
+  float *ptr;
+  int64_t stride_b, stride_h, stride_t;
+} dk_rowvec;
+
+/* CSR (or CSC) look-up table in device memory.  ptr[h][r], ptr[h][r+1] bound
+ * the entries of row block r; entry e is idx[h][e * entry_width] (and the
+ * micro_M value at +1 when entry_width == 2).  num_heads is 1 (shared), the
+ * number of kv heads, or the number of q heads.  Mirrors the tuples
+ * (layout_crow, layout_col, block_m, block_n) of dkernel/interface.py:207-208. */
+typedef struct dk_lut {
+  const int32_t *ptr;
+  const int32_t *idx;
+  int64_t ptr_stride_h, idx_stride_h;
+  int32_t entry_width;
+  int32_t num_heads;
+  int32_t num_rows;    /* row blocks (ptr has num_rows + 1 entries per head) */
+  int32_t block_rows;  /* tokens per row block of this table */
+  int32_t block_cols;  /* tokens per listed entry */
+} dk_lut;
+
+/* Sequence geometry.  With all four pointers NULL every sequence has
+ * q_len = max_q_len and k_len = max_k_len starting at token 0.  Otherwise the
+ * arrays (device memory, int32, `batch` entries) give the first token and the
+ * end (exclusive) of each sequence's queries and keys inside the token
+ * dimension; query tokens are the LAST q_len positions of the sequence when
+ * causal (past_len = k_len - q_len), positions counted from the first real
+ * token.  Mirrors q/k_batch_starts/ends of
+ * dkernel/ops/sparse_attn_inference.py:431-434,503-507. */
+typedef struct dk_seqs {
+  int32_t batch;
+  int32_t max_q_len; /* extent of the q token dimension (total tokens when packed) */
+  int32_t max_k_len;
+  int32_t packed;    /* 1: sequences share one token dimension (3-D inputs) */
+  const int32_t *q_starts, *q_ends, *k_starts, *k_ends;
+} dk_seqs;
+
+/* Forward: O = softmax(mask(Q K^T * sm_scale)) V over the K/V blocks listed in
+ * the CSR table, token-causal when `causal`.  lse.ptr may be NULL.  Rows with
+ * no visible key give O = 0, LSE = -inf.  Tokens outside [q_start, q_end) are
+ * not written.  Replaces the launches of _sparse_fwd_kernel
+ * (dkernel/ops/sparse_attn_fwd.py:519-546) and _fwd_kernel_batch_inference
+ * (dkernel/ops/sparse_attn_inference.py:113-145, :245-285). */
+typedef struct dk_fwd_args {
+  dk_tensor q, k, v, o;
+  dk_rowvec lse; /* natural log */
+  dk_lut csr;
+  dk_seqs seqs;
+  int32_t num_q_heads, num_kv_heads, head_dim;
+  int32_t dtype;  /* enum dk_dtype, of q/k/v/o */
+  int32_t causal;
+  int32_t impl;   /* enum dk_impl */
+  float sm_scale;
+  void *workspace;        /* device scratch for split-KV decode, may be NULL */
+  size_t workspace_bytes;
+  void *stream;           /* hipStream_t */
+} dk_fwd_args;
+
+int dk_fwd(const dk_fwd_args *args);
+/* Scratch that dk_fwd can use for these arguments (0 = none needed). */
+size_t dk_fwd_workspace_bytes(const dk_fwd_args *args);
+
+/* Backward of dk_fwd for equal-length, unpadded sequences (seqs pointers
+ * NULL).  delta is caller scratch of batch * num_q_heads * max_q_len floats.
+ * dlse.ptr may be NULL.  dk/dv are written for every kv head (sum over the q
+ * heads of the group).  Replaces _bwd_preprocess and _sparse_bwd_kernel
+ * launches, dkernel/ops/sparse_attn_bwd.py:781-788, :811-850. */
+typedef struct dk_bwd_args {
+  dk_tensor q, k, v, o, dout, dq, dk, dv;
+  dk_rowvec lse, dlse;
+  float *delta;
+  dk_lut csr, csc;
+  dk_seqs seqs;
+  int32_t num_q_heads, num_kv_heads, head_dim;
+  int32_t dtype;
+  int32_t causal;
+  int32_t impl;
+  float sm_scale;
+  void *stream;
+} dk_bwd_args;
+
+int dk_bwd(const dk_bwd_args *args);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DKERNEL_HIP_H */

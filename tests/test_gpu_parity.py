@@ -1,0 +1,363 @@
+"""GPU parity tests: the HIP path (through the module API and the C ABI)
+against the fp32 dense oracle on identical seeded inputs.  Bar: O and
+dQ/dK/dV within 2e-2 abs/rel, LSE within 1e-3 (fp32 inputs: 2e-4)."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from dkernel_amd import LocalStrideSparseAttention, SparseAttention, combine_attn_partitions, get_sparse_attn_mask
+from dkernel_amd import ops
+from oracle import attention as OA
+from oracle import layout as OL
+from helpers import F32_TOL, LSE_TOL, TOL, assert_close, expand_heads, make_qkv, oracle_fwd
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+@pytest.fixture(params=["generic", "auto"])
+def impl(request):
+    ops.set_impl(request.param)
+    yield request.param
+    ops.set_impl("auto")
+
+
+def _tol(dtype):
+    return F32_TOL if dtype == torch.float32 else TOL
+
+
+def _module(Hq, L, bs, local, vert, **kw):
+    # the class is lru_cached on its constructor arguments
+    return LocalStrideSparseAttention(Hq, L, bs, local, vert, **kw).to(DEV)
+
+
+def _block_mask(Hq, L, bs, local, vert, **kw):
+    kw = {k: v for k, v in kw.items() if k in ("homo_head", "num_kv_heads", "num_dense_heads",
+                                                "head_sliding_offset", "causal")}
+    L = ((L + max(bs, 64) - 1) // max(bs, 64)) * max(bs, 64)
+    return expand_heads(OL.block_mask(Hq, L, bs, local, vert, **kw), Hq)
+
+
+def run_fwd_bwd(B, Hq, Hkv, L, D, dtype, bs=64, local=4, vert=4, seq_dim=1, backward=True,
+                non_contiguous=False, with_dlse=False, **mkw):
+    print(f"case B={B} Hq={Hq} Hkv={Hkv} L={L} D={D} {dtype} bs={bs} local={local} vert={vert} "
+          f"seq_dim={seq_dim} nc={non_contiguous} {mkw}", flush=True)
+    sm_scale = 1.0 / math.sqrt(D)
+    if non_contiguous:
+        q, k, v, do = make_qkv(B, L + 19, L + 19, Hq + 3, Hkv + 3, D, dtype, seq_dim, with_do=True)
+        sl = (slice(None), slice(0, L), slice(0, Hq)) if seq_dim == 1 else (slice(None), slice(0, Hq), slice(0, L))
+        slk = (slice(None), slice(0, L), slice(0, Hkv)) if seq_dim == 1 else (slice(None), slice(0, Hkv), slice(0, L))
+        q, k, v, do = q[sl], k[slk], v[slk], do[sl]
+    else:
+        q, k, v, do = make_qkv(B, L, L, Hq, Hkv, D, dtype, seq_dim, with_do=True)
+    kw = dict(mkw)
+    if Hkv != Hq:
+        kw["num_kv_heads"] = Hkv
+    mod = _module(Hq, L, bs, local, vert, seq_dim=seq_dim, **kw)
+    bm = _block_mask(Hq, L, bs, local, vert, **kw)
+    causal = kw.get("causal", True)
+
+    qo, ko, vo = (x.clone().float().requires_grad_(backward) for x in (q, k, v))
+    ref_o, ref_lse = oracle_fwd(qo, ko, vo, bm, bs, sm_scale, seq_dim, causal=causal)
+
+    qd, kd, vd = (x.to(DEV).requires_grad_(backward) for x in (q, k, v))
+    out, lse = mod(qd, kd, vd, sm_scale, return_lse=True)
+    tol = _tol(dtype)
+    assert out.shape == q.shape and out.dtype == dtype
+    assert_close("O", out, ref_o, **tol)
+    assert_close("LSE", lse, ref_lse, atol=LSE_TOL if dtype != torch.float32 else 1e-4, rtol=0)
+    if not backward:
+        return
+    dlse = None
+    if with_dlse:
+        dlse = torch.randn(ref_lse.shape, generator=torch.Generator().manual_seed(7))
+        (ref_o * do.float()).sum().add((ref_lse * dlse).sum()).backward()
+        (out.float() * do.to(DEV).float()).sum().add((lse * dlse.to(DEV)).sum()).backward()
+    else:
+        ref_o.backward(do.float())
+        out.backward(do.to(DEV))
+    assert_close("dV", vd.grad, vo.grad, **tol)
+    assert_close("dK", kd.grad, ko.grad, **tol)
+    assert_close("dQ", qd.grad, qo.grad, **tol)
+
+
+def test_c0_fp32_plumbing(impl):
+    """B1 L1024 H8 d64 fp32, bs64 local4 vert4, heterogeneous heads, LSE."""
+    run_fwd_bwd(1, 8, 8, 1024, 64, torch.float32, 64, 4, 4, backward=False)
+
+
+@pytest.mark.parametrize("dtype,D,bs", [
+    (torch.bfloat16, 128, 64), (torch.float16, 64, 64), (torch.float32, 64, 64),
+    (torch.bfloat16, 256, 32), (torch.bfloat16, 128, 16), (torch.bfloat16, 64, 128),
+])
+def test_dims_dtypes_block_sizes(impl, dtype, D, bs):
+    run_fwd_bwd(2, 4, 4, 512, D, dtype, bs, 2, 4)
+
+
+@pytest.mark.parametrize("D,dtype", [(48, torch.float32), (96, torch.bfloat16), (160, torch.bfloat16),
+                                     (192, torch.float16)])
+def test_dims_not_power_of_two(impl, D, dtype):
+    run_fwd_bwd(1, 2, 2, 384, D, dtype, 64, 2, 3, homo_head=(D < 100))
+
+
+@pytest.mark.parametrize("L", [15, 100, 1028, 777])
+def test_ragged_lengths(impl, L):
+    run_fwd_bwd(2, 4, 4, L, 128, torch.bfloat16, 64 if L != 1028 else 32, 2, 4)
+
+
+def test_gqa(impl):
+    run_fwd_bwd(2, 8, 2, 512, 128, torch.bfloat16, 64, 3, 4)
+
+
+def test_patterns(impl):
+    run_fwd_bwd(1, 8, 8, 1024, 128, torch.bfloat16, 64, 10, 3)
+    run_fwd_bwd(1, 8, 8, 1024, 128, torch.bfloat16, 64, 1, 8)
+    run_fwd_bwd(1, 8, 8, 1024, 128, torch.bfloat16, 64, 8, 1)
+    run_fwd_bwd(1, 8, 8, 1024, 128, torch.bfloat16, 64, 4, 4, num_dense_heads=2)
+    run_fwd_bwd(1, 8, 8, 1024, 128, torch.bfloat16, 64, 4, 4, homo_head=True)
+    run_fwd_bwd(1, 8, 8, 1024, 128, torch.bfloat16, 64, 2, 8, head_sliding_offset=3)
+
+
+def test_seq_dim_and_non_contiguous(impl):
+    run_fwd_bwd(2, 4, 4, 512, 128, torch.bfloat16, 64, seq_dim=2)
+    run_fwd_bwd(2, 4, 4, 512, 128, torch.bfloat16, 64, seq_dim=1, non_contiguous=True)
+    run_fwd_bwd(2, 4, 4, 512, 128, torch.bfloat16, 64, seq_dim=2, non_contiguous=True)
+
+
+def test_noncausal(impl):
+    run_fwd_bwd(1, 2, 2, 1024, 64, torch.float16, 64, 4, 8, causal=False)
+    run_fwd_bwd(1, 1, 1, 1024, 64, torch.float16, 32, 4, 10000, causal=False)
+
+
+@pytest.mark.parametrize("bs,bm,bn", [(16, 16, 16), (16, 128, 16), (64, 128, 32), (16, 64, 16)])
+def test_kernel_tile_sizes(impl, bs, bm, bn):
+    run_fwd_bwd(1, 2, 2, 1024, 128, torch.bfloat16, bs, 2, 4, block_m=bm, block_n=bn)
+    run_fwd_bwd(1, 2, 2, 1024, 128, torch.bfloat16, bs, 1, 4, block_m=bm, block_n=bn)
+
+
+def test_grad_through_lse(impl):
+    run_fwd_bwd(1, 4, 4, 512, 64, torch.float32, 64, 2, 4, with_dlse=True)
+    run_fwd_bwd(1, 4, 2, 512, 128, torch.bfloat16, 64, 2, 4, with_dlse=True)
+
+
+def test_packed_qkv_and_kv(impl):
+    B, H, L, D = 2, 4, 512, 128
+    q, k, v, do = make_qkv(B, L, L, H, H, D, torch.bfloat16, 1, with_do=True)
+    mod = _module(H, L, 64, 2, 4)
+    qd, kd, vd = (x.to(DEV).requires_grad_() for x in (q, k, v))
+    mod(qd, kd, vd).backward(do.to(DEV))
+    qkv = torch.cat([q, k, v], dim=2).to(DEV).requires_grad_()
+    out = mod(qkv, split_qkv=lambda x: x.chunk(3, dim=2))
+    out.backward(do.to(DEV))
+    dq, dk, dv = qkv.grad.chunk(3, dim=2)
+    assert torch.equal(dq, qd.grad) and torch.equal(dk, kd.grad) and torch.equal(dv, vd.grad)
+    kv = torch.cat([k, v], dim=2).to(DEV).requires_grad_()
+    q2 = q.to(DEV).requires_grad_()
+    mod(q2, kv, split_qkv=lambda x: x.chunk(2, dim=2)).backward(do.to(DEV))
+    dk, dv = kv.grad.chunk(2, dim=2)
+    assert torch.equal(q2.grad, qd.grad) and torch.equal(dk, kd.grad) and torch.equal(dv, vd.grad)
+
+
+# ----------------------------------------------------------------------------
+# inference: paddings, packed variable length, decode
+# ----------------------------------------------------------------------------
+
+def _seq_oracle(q, k, v, bm, bs, sm_scale, causal=True):
+    """One sequence, (L, H, D) tensors, queries = last positions of the keys."""
+    mask = OA.sequence_token_mask(bm, bs, q.shape[0], k.shape[0], causal=causal)
+    o, lse = OA.dense_attention(q[None], k[None], v[None], torch.from_numpy(mask), sm_scale, seq_dim=1)
+    return o[0], lse[0]
+
+
+@pytest.mark.parametrize("seq_dim,bs,dtype,homo", [(1, 64, torch.bfloat16, False), (2, 16, torch.float16, True)])
+def test_left_padded_prefill(impl, seq_dim, bs, dtype, homo):
+    B, Hq, Hkv, L, D = 3, 4, 2, 640, 128
+    sm = 1 / math.sqrt(D)
+    q, k, v = make_qkv(B, L, L, Hq, Hkv, D, dtype, 1)
+    lens = [640, 333, 1]
+    mod = _module(Hq, 1024, bs, 2, 4, num_kv_heads=None if homo else Hkv, homo_head=homo, seq_dim=seq_dim)
+    bm = _block_mask(Hq, 1024, bs, 2, 4, num_kv_heads=None if homo else Hkv, homo_head=homo)
+    qp, kp, vp = (torch.zeros_like(x) for x in (q, k, v))
+    for i, l in enumerate(lens):
+        qp[i, L - l:], kp[i, L - l:], vp[i, L - l:] = q[i, :l], k[i, :l], v[i, :l]
+    tr = (lambda x: x.transpose(1, 2)) if seq_dim == 2 else (lambda x: x)
+    out, lse = mod(tr(qp).to(DEV), tr(kp).to(DEV), tr(vp).to(DEV), sm,
+                   left_paddings=torch.tensor([L - l for l in lens]), return_lse=True)
+    out = tr(out)
+    for i, l in enumerate(lens):
+        ro, rl = _seq_oracle(q[i, :l], k[i, :l], v[i, :l], bm, bs, sm)
+        assert_close(f"O[{i}]", out[i, L - l:], ro, **TOL)
+        assert_close(f"LSE[{i}]", lse[i, :, L - l:], rl, atol=LSE_TOL, rtol=0)
+        assert (out[i, :L - l] == 0).all() and torch.isinf(lse[i, :, :L - l]).all()
+
+
+def test_right_padded_prefill(impl):
+    B, H, L, D, bs = 2, 4, 512, 128, 64
+    sm = 1 / math.sqrt(D)
+    q, k, v = make_qkv(B, L, L, H, H, D, torch.bfloat16, 2)
+    lens = [421, 77]
+    mod = _module(H, 1024, bs, 2, 4, seq_dim=2)
+    bm = _block_mask(H, 1024, bs, 2, 4)
+    out = mod(q.to(DEV), k.to(DEV), v.to(DEV), sm, seqlens=torch.tensor(lens))
+    for i, l in enumerate(lens):
+        ro, _ = _seq_oracle(q[i, :, :l].transpose(0, 1), k[i, :, :l].transpose(0, 1),
+                            v[i, :, :l].transpose(0, 1), bm, bs, sm)
+        assert_close(f"O[{i}]", out[i, :, :l].transpose(0, 1), ro, **TOL)
+        assert (out[i, :, l:] == 0).all()
+
+
+@pytest.mark.parametrize("bs,block_m,left", [(64, None, True), (32, None, True), (16, 128, False), (64, None, False)])
+def test_decode(impl, bs, block_m, left):
+    """One new token per sequence over left-padded / right-padded / unpadded KV, GQA."""
+    B, Hq, Hkv, Lmax, D = 4, 8, 2, 2048, 128
+    sm = 1 / math.sqrt(D)
+    q, k, v = make_qkv(B, 1, Lmax, Hq, Hkv, D, torch.bfloat16, 1)
+    lens = [64 * 21 + 12, 2048, 1, 64 * 5]
+    kw = dict(num_kv_heads=Hkv)
+    if block_m:
+        kw["block_m"] = block_m
+    mod = _module(Hq, Lmax, bs, 2, 4, **kw)
+    bm = _block_mask(Hq, Lmax, bs, 2, 4, num_kv_heads=Hkv)
+    kp, vp = torch.zeros_like(k), torch.zeros_like(v)
+    for i, l in enumerate(lens):
+        if left:
+            kp[i, Lmax - l:], vp[i, Lmax - l:] = k[i, :l], v[i, :l]
+        else:
+            kp[i, :l], vp[i, :l] = k[i, :l], v[i, :l]
+    extra = dict(left_paddings=torch.tensor([Lmax - l for l in lens])) if left else dict(seqlens=torch.tensor(lens))
+    out, lse = mod(q.to(DEV), kp.to(DEV), vp.to(DEV), sm, return_lse=True, **extra)
+    for i, l in enumerate(lens):
+        ro, rl = _seq_oracle(q[i], k[i, :l], v[i, :l], bm, bs, sm)
+        assert_close(f"O[{i}]", out[i], ro, **TOL)
+        assert_close(f"LSE[{i}]", lse[i], rl, atol=LSE_TOL, rtol=0)
+    # unpadded decode through the training entry (q_len 1 < k_len)
+    l = lens[0]
+    out2 = mod(q[:1].to(DEV), k[:1, :l].to(DEV).contiguous(), v[:1, :l].to(DEV).contiguous(), sm)
+    ro, _ = _seq_oracle(q[0], k[0, :l], v[0, :l], bm, bs, sm)
+    assert_close("O unpadded", out2[0], ro, **TOL)
+
+
+def test_packed_varlen_prefill_and_decode(impl):
+    Hq, Hkv, D, bs = 4, 2, 128, 32
+    sm = 1 / math.sqrt(D)
+    lens = [300, 1, 64, 517, 129]
+    T = sum(lens)
+    g = torch.Generator().manual_seed(20)
+    q, k, v = (torch.randn(T, h, D, generator=g).to(torch.bfloat16) for h in (Hq, Hkv, Hkv))
+    cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32)
+    mod = _module(Hq, 1024, bs, 2, 4, num_kv_heads=Hkv)
+    bm = _block_mask(Hq, 1024, bs, 2, 4, num_kv_heads=Hkv)
+    out, lse = mod(q.to(DEV), k.to(DEV), v.to(DEV), sm, cu_seqlen_k=cu.to(DEV), return_lse=True)
+    assert lse.shape == (Hq, T)
+    for i, l in enumerate(lens):
+        s, e = int(cu[i]), int(cu[i + 1])
+        ro, rl = _seq_oracle(q[s:e], k[s:e], v[s:e], bm, bs, sm)
+        assert_close(f"O[{i}]", out[s:e], ro, **TOL)
+        assert_close(f"LSE[{i}]", lse[:, s:e], rl, atol=LSE_TOL, rtol=0)
+    # decode: one query token per sequence (cu_seqlen_q defaults to arange)
+    qd = torch.randn(len(lens), Hq, D, generator=g).to(torch.bfloat16)
+    outd = mod(qd.to(DEV), k.to(DEV), v.to(DEV), sm, cu_seqlen_k=cu.to(DEV))
+    for i, l in enumerate(lens):
+        s, e = int(cu[i]), int(cu[i + 1])
+        ro, _ = _seq_oracle(qd[i:i + 1], k[s:e], v[s:e], bm, bs, sm)
+        assert_close(f"Od[{i}]", outd[i:i + 1], ro, **TOL)
+    # chunked prefill: the last q_len tokens of each sequence
+    qlens = [100, 1, 64, 17, 129]
+    cuq = torch.tensor([0] + list(np.cumsum(qlens)), dtype=torch.int32)
+    qc = torch.cat([q[int(cu[i + 1]) - ql:int(cu[i + 1])] for i, ql in enumerate(qlens)])
+    outc = mod(qc.to(DEV), k.to(DEV), v.to(DEV), sm, cu_seqlen_k=cu.to(DEV), cu_seqlen_q=cuq.to(DEV))
+    for i, ql in enumerate(qlens):
+        assert_close(f"Oc[{i}]", outc[int(cuq[i]):int(cuq[i + 1])], out[int(cu[i + 1]) - ql:int(cu[i + 1])].cpu(),
+                     atol=1e-2, rtol=1e-2)
+
+
+def test_c4_user_pattern_varlen_partitions(impl):
+    """A reduced copy of the user-pattern configuration: per-head Bernoulli
+    block pattern (diagonal forced, lower triangular), packed sequences, LSE,
+    K/V columns split in 2 partitions merged with combine_attn_partitions."""
+    H, D, bs, nb = 4, 128, 64, 32
+    sm = 1 / math.sqrt(D)
+    g = torch.Generator().manual_seed(20)
+    pat = (torch.rand(H, nb, nb, generator=g) < 0.2)
+    pat |= torch.eye(nb, dtype=torch.bool)[None]
+    pat = torch.tril(pat.to(torch.uint8))
+    lens = [512, 700, 64, 333]
+    T = sum(lens)
+    q, k, v = (torch.randn(T, H, D, generator=g).to(torch.bfloat16) for _ in range(3))
+    cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32).to(DEV)
+    full = SparseAttention(bs, pat).to(DEV)
+    c = 6
+    pa, pb = pat.clone(), pat.clone()
+    pa[:, :, c:] = 0
+    pb[:, :, :c] = 0
+    import warnings
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        part_a, part_b = SparseAttention(bs, pa).to(DEV), SparseAttention(bs, pb).to(DEV)
+    args = (q.to(DEV), k.to(DEV), v.to(DEV), sm)
+    o_full, lse_full = full(*args, cu_seqlen_k=cu, return_lse=True)
+    ra = part_a(*args, cu_seqlen_k=cu, return_lse=True)
+    rb = part_b(*args, cu_seqlen_k=cu, return_lse=True)
+    assert torch.isinf(rb[1]).any() and (rb[0][torch.isinf(rb[1]).transpose(0, 1)] == 0).all()
+    merged = combine_attn_partitions(ra, rb)
+    assert_close("combine vs unpartitioned", merged, o_full.cpu(), atol=1e-2, rtol=1e-2)
+    lse_merged = torch.logaddexp(ra[1], rb[1])
+    assert_close("lse merge", lse_merged, lse_full.cpu(), atol=LSE_TOL, rtol=0)
+    s = 0
+    for l in lens:
+        ro, rl = _seq_oracle(q[s:s + l], k[s:s + l], v[s:s + l], pat.numpy(), bs, sm)
+        assert_close("O vs oracle", merged[s:s + l], ro, **TOL)
+        assert_close("LSE vs oracle", lse_full[:, s:s + l], rl, atol=LSE_TOL, rtol=0)
+        s += l
+
+
+def test_seq_partition_with_backward(impl):
+    """Context-parallel emulation in one process (reference:
+    tests/test_seq_partition.py): q chunks x kv partitions, non-square masks,
+    merge with combine_attn_partitions, gradients through the LSE."""
+    B, H, L, D, bs, parts = 1, 3, 1024, 64, 32, 4
+    dtype = torch.float16
+    q, k, v, do = make_qkv(B, L, L, H, H, D, dtype, 2, with_do=True)
+    qd, kd, vd = (x.to(DEV).requires_grad_() for x in (q, k, v))
+    chunk = L // parts
+    outs = []
+    for qc in range(parts):
+        pieces = []
+        for kc in range(qc + 1):
+            _, bmask, _ = get_sparse_attn_mask(H, chunk, bs, 4, 4, dtype=dtype, q_start_position=qc * chunk,
+                                               kv_start_position=kc * chunk, kv_seqlen=chunk)
+            layer = SparseAttention(bs, bmask, seq_dim=2, causal=(kc == qc)).to(DEV)
+            pieces.append(layer(qd[:, :, qc * chunk:(qc + 1) * chunk], kd[:, :, kc * chunk:(kc + 1) * chunk],
+                                vd[:, :, kc * chunk:(kc + 1) * chunk], return_lse=True))
+        outs.append(pieces[0][0] if len(pieces) == 1 else combine_attn_partitions(*pieces, hdim=1))
+    out = torch.cat(outs, dim=2)
+    out.backward(do.to(DEV))
+    bm = OL.block_mask(H, L, bs, 4, 4)
+    qo, ko, vo = (x.clone().float().requires_grad_() for x in (q, k, v))
+    ref, _ = oracle_fwd(qo, ko, vo, bm, bs, 1 / math.sqrt(D), seq_dim=2)
+    ref.backward(do.float())
+    assert_close("O", out, ref, **TOL)
+    assert_close("dQ", qd.grad, qo.grad, **TOL)
+    assert_close("dK", kd.grad, ko.grad, **TOL)
+    assert_close("dV", vd.grad, vo.grad, **TOL)
+
+
+def test_error_paths(impl):
+    mod = _module(4, 512, 64, 2, 4)
+    x = torch.zeros(1, 1024, 4, 128, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(AssertionError, match="larger than the maximum length"):
+        mod(x, x, x)
+    y = torch.zeros(1, 256, 4, 128, dtype=torch.bfloat16, device=DEV, requires_grad=True)
+    out = mod(y, y, y, left_paddings=torch.zeros(1, dtype=torch.int32))
+    with pytest.raises(AssertionError, match="does not support paddings"):
+        out.sum().backward()
+    z = torch.zeros(1, 256, 3, 128, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(AssertionError, match="number of heads in the sparse pattern"):
+        mod(z, z, z)
+    with pytest.raises(AssertionError, match="q length can only 1"):
+        mod(y[:, :7], y, y, seqlens=torch.tensor([5]))
+    # empty batch is a no-op
+    e = torch.zeros(0, 256, 4, 128, dtype=torch.bfloat16, device=DEV)
+    assert mod(e, e, e).shape == e.shape

@@ -1,0 +1,180 @@
+"""CPU tests of the product's host side: the C++ look-up-table builder behind
+the C ABI against the golden fixtures and the oracle (bit-exact), the module
+constructors, and the C-ABI surface (library loads, every declared symbol is
+exported).  No compute call is made without a GPU."""
+import ctypes
+import os
+import re
+import warnings
+import zlib
+
+import numpy as np
+import pytest
+import torch
+
+import dkernel_amd
+from dkernel_amd import _lib, utils as U
+from dkernel_amd.interface import LocalStrideSparseAttention, SparseAttention, combine_attn_partitions
+from oracle import layout as OL
+from conftest import ROOT, mask_kwargs
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "dkernel_hip.h")).read()
+    declared = set(re.findall(r"\b(dk_[a-z_0-9]+)\s*\(", header))
+    assert declared == set(_lib.SYMBOLS), declared ^ set(_lib.SYMBOLS)
+    handle = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared:
+        assert hasattr(handle, name), name
+    assert _lib.lib().dk_version() >= 100
+    assert _lib.lib().dk_last_error() is not None
+
+
+def test_struct_sizes_match_header():
+    # natural alignment on x86-64: catches a field added on one side only
+    assert ctypes.sizeof(_lib.Tensor) == 32 and ctypes.sizeof(_lib.RowVec) == 32
+    assert ctypes.sizeof(_lib.Lut) == 56 and ctypes.sizeof(_lib.Seqs) == 48
+    assert ctypes.sizeof(_lib.FwdArgs) == 4 * 32 + 32 + 56 + 48 + 7 * 4 + 4 + 3 * 8
+    assert ctypes.sizeof(_lib.BwdArgs) == 8 * 32 + 2 * 32 + 8 + 2 * 56 + 48 + 7 * 4 + 4 + 8
+
+
+def test_mask_and_luts_match_fixtures(lut_fixtures):
+    z, meta = lut_fixtures
+    for name, kw in meta["mask"].items():
+        (crow, col), bm, _ = U.get_sparse_attn_mask(dtype=torch.uint8, **mask_kwargs(kw))
+        assert bm.dtype == torch.uint8 and crow.dtype == torch.int32 and col.dtype == torch.int32
+        assert np.array_equal(bm.cpu().numpy(), z[f"mask/{name}/block_mask"]), name
+        assert np.array_equal(crow.cpu().numpy(), z[f"mask/{name}/crow"]), name
+        assert np.array_equal(col.cpu().numpy(), z[f"mask/{name}/col"]), name
+        ccol, row = U.dense_to_ccol_row(bm)
+        assert np.array_equal(ccol.cpu().numpy(), z[f"mask/{name}/ccol"]), name
+        assert np.array_equal(row.cpu().numpy(), z[f"mask/{name}/row"]), name
+        assert U.is_kv_cache_efficient(bm, kw["block_size"], kw["block_size"]) == bool(z[f"mask/{name}/kv_eff"])
+
+
+def test_tile_luts_match_fixtures(lut_fixtures):
+    z, meta = lut_fixtures
+    for name, t in meta["tile"].items():
+        pat = torch.from_numpy(z[f"tile/{name}/pattern"])
+        crow, col = U.merge_split_fwd_kernel_blocks(t["block_size"], pat, t["block_m"], t["block_n"])
+        assert np.array_equal(crow.cpu().numpy(), z[f"tile/{name}/crow"]), name
+        assert np.array_equal(col.cpu().numpy(), z[f"tile/{name}/col"]), name
+
+
+def test_headline_lut(lut_fixtures):
+    z, meta = lut_fixtures
+    (crow, col), bm, _ = U.get_sparse_attn_mask(dtype=torch.uint8, **meta["c1"])
+    ccol, row = U.dense_to_ccol_row(bm)
+    assert np.array_equal(crow.cpu().numpy(), z["c1/crow"]) and np.array_equal(ccol.cpu().numpy(), z["c1/ccol"])
+    crc = [zlib.crc32(np.ascontiguousarray(x.cpu().numpy()).tobytes()) for x in (bm, col, row)]
+    assert crc == list(z["c1/crc"])
+
+
+@pytest.mark.parametrize("kw", [
+    dict(num_heads=8, seqlen=777, block_size=32, local_blocks=3, vert_stride=5, num_kv_heads=4,
+         head_sliding_offset=2, num_dense_heads=1),
+    dict(num_heads=6, seqlen=512, block_size=16, local_blocks=1, vert_stride=7, head_sliding_step=2),
+    dict(num_heads=4, seqlen=320, block_size=64, local_blocks=2, vert_stride=3, causal=False),
+    dict(num_heads=4, seqlen=320, block_size=64, local_blocks=2, vert_stride=3, causal=False,
+         num_dense_heads=2),
+    dict(num_heads=4, seqlen=256, block_size=32, local_blocks=2, vert_stride=3, past_len=100),
+    dict(num_heads=2, seqlen=128, block_size=32, local_blocks=2, vert_stride=3,
+         q_start_position=256, kv_start_position=64, kv_seqlen=320),
+])
+def test_mask_matches_oracle(kw):
+    (crow, col), bm, dense = U.get_sparse_attn_mask(dtype=torch.uint8, return_dense=True, **kw)
+    want = OL.block_mask(**kw)
+    assert np.array_equal(bm.cpu().numpy(), want)
+    ocrow, ocol = OL.csr_from_dense(want)
+    assert np.array_equal(crow.cpu().numpy(), ocrow) and np.array_equal(col.cpu().numpy(), ocol)
+    if "q_start_position" not in kw:
+        full = OL.block_mask(**{k: v for k, v in kw.items() if k != "past_len"})
+        tok = OL.token_mask(full, kw["block_size"], kw["seqlen"], past_len=kw.get("past_len", 0),
+                            causal=kw.get("causal", True))
+        assert np.array_equal(dense.cpu().numpy(), np.broadcast_to(tok, dense.shape))
+
+
+def test_csr_random_and_edge_cases():
+    rng = np.random.default_rng(1)
+    x = torch.from_numpy((rng.random((3, 7, 11)) < 0.4).astype(np.uint8))
+    x[2] = 0
+    for t in (x, x[0], x.transpose(1, 2), x.to(torch.bool), x.to(torch.bfloat16)):
+        crow, col = U.dense_to_crow_col(t)
+        ocrow, ocol = OL.csr_from_dense(t.to(torch.int32).numpy())
+        assert np.array_equal(crow.numpy(), ocrow) and np.array_equal(col.numpy(), ocol)
+    crow, col = U.dense_to_crow_col(torch.zeros(2, 3, 4))      # all empty: zero-width col
+    assert col.shape == (2, 0) and (crow == 0).all()
+    vals = torch.from_numpy(rng.integers(0, 4, (2, 5, 6)).astype(np.int32)) * 16
+    crow, col = U.dense_to_crow_col(vals, include_values=True)
+    ocrow, ocol = OL.csr_from_dense(vals.numpy(), include_values=True)
+    assert np.array_equal(crow.numpy(), ocrow) and np.array_equal(col.numpy(), ocol)
+    assert np.array_equal(U.crow_col_to_dense(*U.dense_to_crow_col(x), dtype=torch.uint8).numpy()[:2],
+                          x.numpy()[:2, :, :U.dense_to_crow_col(x)[1].max() + 1])
+
+
+def test_kv_cache_check_and_warning():
+    rng = np.random.default_rng(3)
+    for _ in range(20):
+        p = np.tril((rng.random((2, 6, 6)) < 0.5).astype(np.uint8))
+        assert U.is_kv_cache_efficient(torch.from_numpy(p), 4, 4) == OL.kv_cache_efficient(p, 4, 4)
+    pat = torch.tril((torch.rand(4, 8, 8, generator=torch.Generator().manual_seed(0)) < 0.3).to(torch.uint8))
+    pat[:, torch.arange(8), torch.arange(8)] = 1
+    with warnings.catch_warnings(record=True) as w:
+        warnings.simplefilter("always")
+        SparseAttention(64, pat)
+    assert any("not efficient for KV cache" in str(x.message) for x in w)
+
+
+def test_module_construction_matches_reference_surface():
+    assert dkernel_amd.__all__ == ["SparseAttention", "LocalStrideSparseAttention",
+                                   "get_sparse_attn_mask", "combine_attn_partitions"]
+    m = LocalStrideSparseAttention(32, 8192, 64, 16, 8, num_kv_heads=8)
+    assert m is LocalStrideSparseAttention(32, 8192, 64, 16, 8, num_kv_heads=8)     # lru_cache
+    assert (m.block_m, m.block_n, m.block_m2, m.block_n2, m.max_seqlen) == (64, 64, 64, 64, 8192)
+    assert m.layout_csr_crow.shape == (32, 129) and m.layout_csr_col.shape == (32, 2768)
+    assert m.layout_csc_ccol.shape == (32, 129) and m.layout_csc_row.shape == (32, 2768)
+    assert all(b.dtype == torch.int32 for b in m.buffers()) and len(m.state_dict()) == 0
+    assert int(m.layout_csr_crow[:, -1].sum()) == 87008
+    # homogeneous pattern: one head with stride 0
+    h = LocalStrideSparseAttention(8, 1000, 64, 4, 4, homo_head=True)
+    assert h.max_seq_len == 1024 and h.layout_csr_crow.shape[0] == 1 and h.layout_csr_crow.stride(0) == 0
+    # head slicing for head parallelism
+    full = LocalStrideSparseAttention(8, 1024, 64, 2, 8)
+    part = LocalStrideSparseAttention(8, 1024, 64, 2, 8, active_head_range=(2, 6))
+    assert torch.equal(part.layout_csr_crow, full.layout_csr_crow[2:6])
+    # merged-q table carries (col, micro_M)
+    mq = LocalStrideSparseAttention(2, 512, 16, 2, 4, block_m=128, block_n=16)
+    assert mq.layout_csr_col.dim() == 3 and mq.layout_csr_col.shape[-1] == 2
+    with pytest.raises(AssertionError):
+        SparseAttention(24, torch.ones(4, 4))
+    with pytest.raises(AssertionError):
+        LocalStrideSparseAttention(8, 1024, 64, 0, 8)
+
+
+def test_cpu_tensors_are_refused_loudly():
+    m = LocalStrideSparseAttention(2, 128, 64, 1, 2)
+    x = torch.zeros(1, 128, 2, 64)
+    with pytest.raises(RuntimeError, match="no CPU execution path"):
+        m(x, x, x)
+
+
+def test_combine_matches_closed_form():
+    g = torch.Generator().manual_seed(0)
+    o = [torch.randn(2, 3, 5, 4, generator=g) for _ in range(3)]
+    l = [torch.randn(2, 3, 5, generator=g) for _ in range(3)]
+    l[1][0, 0, 0] = float("-inf")
+    got = combine_attn_partitions(*zip(o, l))
+    w = torch.softmax(torch.stack(l), 0)
+    want = (torch.stack(o) * w[..., None]).sum(0)
+    assert torch.allclose(got, want, atol=1e-6)
+    # (batch, seq, heads, dim) outputs with (batch, heads, seq) log-sum-exps
+    got2 = combine_attn_partitions(*[(x.transpose(1, 2), y) for x, y in zip(o, l)], hdim=2)
+    assert torch.allclose(got2, want.transpose(1, 2), atol=1e-6)
+    # packed (tokens, heads, dim) outputs with (heads, tokens) log-sum-exps
+    got3 = combine_attn_partitions(*[(x[0].transpose(0, 1), y[0]) for x, y in zip(o, l)])
+    assert torch.allclose(got3, want[0].transpose(0, 1), atol=1e-6)
+    # every partition empty for a row -> 0, not NaN
+    l2 = [x.clone() for x in l]
+    for x in l2:
+        x[1, 2, 3] = float("-inf")
+    assert torch.isfinite(combine_attn_partitions(*zip(o, l2))).all()

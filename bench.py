@@ -1,0 +1,201 @@
+"""Benchmark of the block-sparse attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extra]
+
+A step is one causal prefill forward (with LSE) over one synthetic batch of the
+Phi-3-small-style configuration: B=2, L=8192, 32 q heads / 8 kv heads, head_dim
+128, bf16, block 64, 16 local blocks, vertical stride 8.  Inputs are resident
+in HBM before the timed region.  Prints ONE JSON line:
+
+  value     effective (sparse-counted) TFLOP/s = 4*64*64*128 * active blocks / time
+  roofline  the forward kernel against the dense bf16 MFMA peak, from HIP
+            events on the launch stream around the same timed steps
+  cpu_baseline  the reference's dense masked-attention checker (oracle port)
+            timed on this box's host cores on a bounded sample
+  extra     backward (B=1, 32 MHA heads) TFLOP/s and batched-decode us/step
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16, vendor figure
+HBM_PEAK_GBS = 8000.0            # MI355X HBM3E, vendor figure
+BS, LOCAL, VERT, D = 64, 16, 8, 128
+
+
+def block_flops(nnz_blocks, d=D, bs=BS):
+    """QK^T and PV over one bs x bs block, diagonal blocks counted in full."""
+    return 4.0 * bs * bs * d * nnz_blocks
+
+
+def gen(shape, g, dtype):
+    import torch
+    return torch.randn(shape, generator=g, dtype=torch.float32).to(dtype)
+
+
+def time_steps(fn, steps, warmup):
+    """(wall ms per step, HIP-event ms per step) over exactly `steps` calls."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(steps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) * 1e3 / steps
+    return wall, start.elapsed_time(stop) / steps
+
+
+def cpu_baseline(seconds_budget=20.0):
+    """The reference checker's dense masked attention (oracle port) on the host
+    CPU, on a bounded sample of the same workload: whole heads of one batch
+    element at L=8192, d=128, bf16 inputs, until the budget is spent."""
+    import torch
+    from oracle import attention as OA
+    from oracle import layout as OL
+    cores = os.cpu_count() or 1
+    # the GPU box caps worker pools at 16 threads per GPU
+    threads = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)), 16)
+    torch.set_num_threads(threads)
+    L, H, Hkv = 8192, 32, 8
+    g = torch.Generator().manual_seed(20)
+    bm = OL.block_mask(H, L, BS, LOCAL, VERT, num_kv_heads=Hkv)
+    sm = 1.0 / math.sqrt(D)
+    done_blocks, heads, t_total = 0, 0, 0.0
+    tril = torch.tril(torch.ones(L, L, dtype=torch.bool))
+    while t_total < seconds_budget and heads < H:
+        h = heads
+        q, k, v = (gen((1, 1, L, D), g, torch.bfloat16) for _ in range(3))
+        mask = torch.from_numpy(bm[h]).bool().repeat_interleave(BS, 0).repeat_interleave(BS, 1) & tril
+        t0 = time.perf_counter()
+        OA.reference_style_attention(q, k, v, mask[None, None], sm, seq_dim=2)
+        t_total += time.perf_counter() - t0
+        done_blocks += int(bm[h].sum())
+        heads += 1
+    return {
+        "value": round(block_flops(done_blocks) / t_total / 1e12, 5),
+        "unit": "TFLOP/s (effective, sparse-counted)",
+        "cores": threads,
+        "kind": "port",
+        "sample": f"{heads} of 64 (batch, head) pairs at L=8192 d=128 bf16, dense masked torch attention, "
+                  f"{t_total:.1f} s",
+        "dense_tflops": round(4.0 * L * L * D * heads / t_total / 1e12, 5),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=25)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="skip backward / decode figures")
+    ap.add_argument("--impl", default="auto", choices=["auto", "generic", "mfma"])
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: the path has no cross-GPU component in this build "
+              "(heads and KV partitions shard without communication; see DESIGN.md). Use --gpus 1.",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from dkernel_amd import LocalStrideSparseAttention, ops
+    ops.set_impl(args.impl)
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+    g = torch.Generator().manual_seed(20)
+    sm = 1.0 / math.sqrt(D)
+
+    # ---- C1: prefill forward -------------------------------------------------
+    B, L, Hq, Hkv = 2, 8192, 32, 8
+    mod = LocalStrideSparseAttention(Hq, L, BS, LOCAL, VERT, num_kv_heads=Hkv).to(dev)
+    nnz = int(mod.layout_csr_crow[:, -1].sum().item())      # 87008 per batch element
+    q = gen((B, L, Hq, D), g, torch.bfloat16).to(dev)
+    k = gen((B, L, Hkv, D), g, torch.bfloat16).to(dev)
+    v = gen((B, L, Hkv, D), g, torch.bfloat16).to(dev)
+    with torch.no_grad():
+        wall_ms, ev_ms = time_steps(lambda: mod(q, k, v, sm, return_lse=True), args.steps, args.warmup)
+    flops = block_flops(nnz) * B
+    value = flops / (wall_ms * 1e-3) / 1e12
+    achieved = flops / (ev_ms * 1e-3) / 1e12
+
+    out = {
+        "metric": "effective fwd TFLOP/s, causal block-sparse prefill, L=8192 d=128 bf16, 1 MI355X",
+        "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall_ms, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "prefill fwd + LSE: B=2 L=8192 Hq=32 Hkv=8 d=128 bf16, block 64, "
+                               "local 16, vert 8, heterogeneous heads, causal",
+                   "active_blocks_per_batch": nnz, "flop_per_step": flops, "impl": args.impl},
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_BF16_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4),
+                     "traffic": None, "kernel_ms": round(ev_ms, 4)},
+    }
+    del q, k, v
+
+    if not args.no_extra:
+        extra = {}
+        # ---- C2: backward, B=1, 32 MHA heads ---------------------------------
+        mod2 = LocalStrideSparseAttention(32, L, BS, LOCAL, VERT).to(dev)
+        nnz2 = int(mod2.layout_csr_crow[:, -1].sum().item())
+        q2, k2, v2, do2 = (gen((1, L, 32, D), g, torch.bfloat16).to(dev) for _ in range(4))
+        q2.requires_grad_(), k2.requires_grad_(), v2.requires_grad_()
+        o2 = mod2(q2, k2, v2, sm)
+
+        def bwd():
+            torch.autograd.grad(o2, (q2, k2, v2), do2, retain_graph=True)
+        steps2 = max(5, args.steps // 4)
+        w2, e2 = time_steps(bwd, steps2, max(2, args.warmup // 4))
+        with torch.no_grad():
+            wf, ef = time_steps(lambda: mod2(q2, k2, v2, sm), steps2, 2)
+        extra["bwd"] = {"workload": "dQ,dK,dV: B=1 L=8192 H=32 (MHA) d=128 bf16, same pattern",
+                        "tflops": round(2.5 * block_flops(nnz2) / (e2 * 1e-3) / 1e12, 2),
+                        "ms": round(e2, 4), "frac_of_mfma_peak":
+                        round(2.5 * block_flops(nnz2) / (e2 * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+                        "fwd_mha_tflops": round(block_flops(nnz2) / (ef * 1e-3) / 1e12, 2)}
+        del q2, k2, v2, do2, o2
+        # ---- C3: batched decode over left-padded KV --------------------------
+        nseq, Lmax = 32, 8192
+        lens = torch.randint(1024, 8193, (nseq,), generator=g)
+        kd = torch.zeros((nseq, Lmax, Hkv, D), dtype=torch.bfloat16)
+        vd = torch.zeros_like(kd)
+        for i, l in enumerate(lens.tolist()):
+            kd[i, Lmax - l:] = gen((l, Hkv, D), g, torch.bfloat16)
+            vd[i, Lmax - l:] = gen((l, Hkv, D), g, torch.bfloat16)
+        kd, vd = kd.to(dev), vd.to(dev)
+        qd = gen((nseq, 1, Hq, D), g, torch.bfloat16).to(dev)
+        left = (Lmax - lens).to(torch.int32).to(dev)
+        # algorithmic bytes: K and V of every attended token, once per kv head
+        byts = 0
+        for l in lens.tolist():
+            r = (l - 1) // BS
+            for kvh in range(Hkv):
+                nblk = min(r + 1, LOCAL) + sum(1 for j in range(0, max(r - LOCAL + 1, 0)) if (j + kvh) % VERT == 0)
+                byts += (BS * (nblk - 1) + ((l - 1) % BS + 1)) * D * 2 * 2
+        with torch.no_grad():
+            wd, ed = time_steps(lambda: mod(qd, kd, vd, sm, left_paddings=left), args.steps, args.warmup)
+        extra["decode"] = {"workload": "32 seqs x 1 token, Hq=32 Hkv=8 d=128 bf16, KV len U[1024,8192] left-padded",
+                           "us_per_step": round(wd * 1e3, 2), "kernel_us": round(ed * 1e3, 2),
+                           "algorithmic_MB": round(byts / 1e6, 2),
+                           "achieved_GBs": round(byts / (ed * 1e-3) / 1e9, 1),
+                           "frac_of_hbm_peak": round(byts / (ed * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+        out["extra"] = extra
+
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

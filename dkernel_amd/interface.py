@@ -19,6 +19,19 @@ from .utils import (dense_to_ccol_row, get_sparse_attn_mask, is_kv_cache_efficie
                     merge_split_fwd_kernel_blocks, multiple_of, verify_sparse_pattern, zero_stride)
 
 
+def _identical_head_run(pattern: Tensor) -> int:
+    """Largest g dividing the number of pattern heads such that every run of g
+    consecutive heads holds one and the same pattern."""
+    H = pattern.size(0)
+    p = pattern.cpu()
+    for g in (8, 4, 2):
+        if H % g == 0 and H >= g:
+            grouped = p.reshape(H // g, g, *p.shape[1:])
+            if bool((grouped == grouped[:, :1]).all()):
+                return g
+    return 1
+
+
 class SparseAttention(torch.nn.Module):
     """Block-sparse attention over a user-given block pattern.
 
@@ -83,6 +96,9 @@ class SparseAttention(torch.nn.Module):
         self.kwargs = copy.copy(kwargs)
         self.kwargs["max_seqlen"] = self.max_seqlen
         self.kwargs['causal'] = causal
+        # q heads whose patterns are identical (a GQA group) can share K/V tiles on chip
+        self.lut_group = _identical_head_run(sparse_pattern)
+        self.kwargs['lut_group'] = self.lut_group
 
         if not causal:
             # merged q tiles are a causal-only optimisation

@@ -62,7 +62,7 @@ def _rowvec(x: Optional[Tensor], strides=None) -> _lib.RowVec:
     return _lib.RowVec(x.data_ptr(), sb, sh, st)
 
 
-def _lut(layout: Tuple[Tensor, Tensor, int, int], device) -> _lib.Lut:
+def _lut(layout: Tuple[Tensor, Tensor, int, int], device, group: int = 1) -> _lib.Lut:
     ptr, idx, block_rows, block_cols = layout
     assert ptr.dtype == torch.int32 and idx.dtype == torch.int32
     assert ptr.device == device and idx.device == device, \
@@ -77,7 +77,7 @@ def _lut(layout: Tuple[Tensor, Tensor, int, int], device) -> _lib.Lut:
     else:
         assert idx.stride(-1) == 1 or idx.size(-1) <= 1
     return _lib.Lut(ptr.data_ptr(), idx.data_ptr(), ptr.stride(0), idx.stride(0), width,
-                    ptr.size(0), ptr.size(1) - 1, int(block_rows), int(block_cols))
+                    ptr.size(0), ptr.size(1) - 1, int(block_rows), int(block_cols), int(group))
 
 
 def _stream() -> C.c_void_p:
@@ -103,7 +103,8 @@ def _forward(ctx, q: Tensor, k: Tensor, v: Tensor, sm_scale: float,
              max_seqlen: Optional[int] = None,
              return_lse: bool = False,
              causal=True,
-             split_qkv=None) -> Tuple[Tensor, Optional[Tensor]]:
+             split_qkv=None,
+             lut_group: int = 1) -> Tuple[Tensor, Optional[Tensor]]:
     """Unpadded 4-D forward (training, prefill, single-token decode).
     Reference: dkernel/ops/sparse_attn_fwd.py:383-567.  `d_splits` is accepted
     and ignored (a Triton shared-memory workaround)."""
@@ -129,7 +130,7 @@ def _forward(ctx, q: Tensor, k: Tensor, v: Tensor, sm_scale: float,
     args = _lib.FwdArgs()
     args.q, args.k, args.v, args.o = (_tensor4(x, hdim, seq_dim) for x in (q, k, v, o))
     args.lse = _rowvec(lse)
-    args.csr = _lut(layout_csr, q.device)
+    args.csr = _lut(layout_csr, q.device, lut_group)
     args.seqs = _lib.Seqs(q.size(0), qlen, klen, 0, None, None, None, None)
     args.num_q_heads, args.num_kv_heads, args.head_dim = num_heads, num_kv_heads, q.size(-1)
     args.dtype, args.causal, args.impl = _DTYPES[q.dtype], int(bool(causal)), _impl
@@ -142,6 +143,7 @@ def _forward(ctx, q: Tensor, k: Tensor, v: Tensor, sm_scale: float,
     ctx.seq_dim = seq_dim
     ctx.hdim = hdim
     ctx.causal = causal
+    ctx.lut_group = lut_group
     return o, (lse if return_lse else None)
 
 
@@ -175,8 +177,8 @@ def _backward(ctx, do: Tensor, dlse: Optional[Tensor],
     else:
         args.dlse = _rowvec(None)
     args.delta = delta.data_ptr()
-    args.csr = _lut(ctx.layout_csr, q.device)
-    args.csc = _lut(ctx.layout_csc, q.device)
+    args.csr = _lut(ctx.layout_csr, q.device, ctx.lut_group)
+    args.csc = _lut(ctx.layout_csc, q.device, ctx.lut_group)
     args.seqs = _lib.Seqs(B, Lq, k.size(seq_dim), 0, None, None, None, None)
     args.num_q_heads, args.num_kv_heads, args.head_dim = Hq, k.size(hdim), q.size(-1)
     args.dtype, args.causal, args.impl = _DTYPES[q.dtype], int(bool(ctx.causal)), _impl
@@ -196,7 +198,8 @@ def padded_sparse_attn(q: Tensor, k: Tensor, v: Tensor, sm_scale: float,
                        out: Optional[Tensor] = None,
                        inference: bool = True,
                        causal: bool = True,
-                       return_lse: bool = False):
+                       return_lse: bool = False,
+                       lut_group: int = 1):
     """4-D inputs with left paddings and / or explicit sequence lengths; q has
     either one token per sequence (decode) or the same padded length as k.
     Reference: dkernel/ops/sparse_attn_inference.py:10-147.  Padding rows of
@@ -242,7 +245,7 @@ def padded_sparse_attn(q: Tensor, k: Tensor, v: Tensor, sm_scale: float,
     args = _lib.FwdArgs()
     args.q, args.k, args.v, args.o = (_tensor4(x, hdim, seq_dim) for x in (q, k, v, out))
     args.lse = _rowvec(lse)
-    args.csr = _lut(sparse_layout, dev)
+    args.csr = _lut(sparse_layout, dev, lut_group)
     args.seqs = _lib.Seqs(batches, q_len, k_len, 0, q_starts.data_ptr(), q_ends.data_ptr(),
                           k_starts.data_ptr(), k_ends.data_ptr())
     args.num_q_heads, args.num_kv_heads, args.head_dim = num_heads, num_kv_heads, head_size
@@ -262,7 +265,8 @@ def varlen_sparse_attn(q: Tensor, k: Tensor, v: Tensor,
                        out: Optional[Tensor] = None,
                        inference: bool = True,
                        causal: bool = True,
-                       return_lse: bool = False):
+                       return_lse: bool = False,
+                       lut_group: int = 1):
     """Packed variable-length inputs (total_tokens, heads, head_dim) with
     cumulative sequence lengths.  Reference:
     dkernel/ops/sparse_attn_inference.py:150-287.  The query tokens of a
@@ -296,7 +300,7 @@ def varlen_sparse_attn(q: Tensor, k: Tensor, v: Tensor,
     args = _lib.FwdArgs()
     args.q, args.k, args.v, args.o = (_tensor3(x) for x in (q, k, v, out))
     args.lse = _rowvec(lse, (0, lse.stride(0), lse.stride(1))) if lse is not None else _rowvec(None)
-    args.csr = _lut(sparse_layout, dev)
+    args.csr = _lut(sparse_layout, dev, lut_group)
     isz = cu_q.element_size()
     args.seqs = _lib.Seqs(batch_size, q.size(0), k.size(0), 1,
                           cu_q.data_ptr(), cu_q.data_ptr() + isz, cu_k.data_ptr(), cu_k.data_ptr() + isz)
@@ -348,6 +352,7 @@ class _sparse_attention(torch.autograd.Function):
         max_seqlen = kwargs.get("max_seqlen", None)
         causal = kwargs.get("causal", True)
         return_lse = kwargs.get("return_lse", False)
+        lut_group = kwargs.get("lut_group", 1)
         lse = None
 
         assert q.dim() in (3, 4)
@@ -364,7 +369,7 @@ class _sparse_attention(torch.autograd.Function):
             ctx.message = "Currently does not suppoort variable length inputs. WIP."
             res = varlen_sparse_attn(q, k, v, inf_kwargs["cu_seqlen_k"], inf_kwargs.get("cu_seqlen_q", None),
                                      sm_scale, layout_csr, max_seqlen=max_seqlen, causal=causal,
-                                     return_lse=return_lse)
+                                     return_lse=return_lse, lut_group=lut_group)
             output, lse = res if return_lse else (res, None)
         else:
             assert k.size(seq_dim) <= max_seqlen, \
@@ -377,14 +382,14 @@ class _sparse_attention(torch.autograd.Function):
                 ctx.message = "Currently does not support paddings in inputs. WIP."
                 res = padded_sparse_attn(q, k, v, sm_scale, layout_csr, left_paddings=left_paddings,
                                          seqlens=seqlens, seq_dim=seq_dim, max_seqlen=max_seqlen,
-                                         causal=causal, return_lse=return_lse)
+                                         causal=causal, return_lse=return_lse, lut_group=lut_group)
                 output, lse = res if return_lse else (res, None)
             else:
                 ctx.support_backward = True
                 ctx.message = ""
                 fwd_kwargs = {k_: v_ for k_, v_ in kwargs.items()
                               if k_ in ("inference", "out", "d_splits", "max_seqlen", "return_lse",
-                                        "causal", "split_qkv")}
+                                        "causal", "split_qkv", "lut_group")}
                 output, lse = _forward(ctx, q, k, v, sm_scale, layout_csr, seq_dim=seq_dim, **fwd_kwargs)
         return output, lse
 

@@ -106,6 +106,8 @@ typedef struct dk_lut {
   int32_t num_rows;    /* row blocks (ptr has num_rows + 1 entries per head) */
   int32_t block_rows;  /* tokens per row block of this table */
   int32_t block_cols;  /* tokens per listed entry */
+  int32_t group;       /* consecutive table heads known to hold identical rows (1 if unknown);
+                          lets heads of a GQA group share K/V tiles inside a workgroup */
 } dk_lut;
 
 /* Sequence geometry.  With all four pointers NULL every sequence has

@@ -33,9 +33,9 @@ def test_library_exports_every_declared_symbol():
 def test_struct_sizes_match_header():
     # natural alignment on x86-64: catches a field added on one side only
     assert ctypes.sizeof(_lib.Tensor) == 32 and ctypes.sizeof(_lib.RowVec) == 32
-    assert ctypes.sizeof(_lib.Lut) == 56 and ctypes.sizeof(_lib.Seqs) == 48
-    assert ctypes.sizeof(_lib.FwdArgs) == 4 * 32 + 32 + 56 + 48 + 7 * 4 + 4 + 3 * 8
-    assert ctypes.sizeof(_lib.BwdArgs) == 8 * 32 + 2 * 32 + 8 + 2 * 56 + 48 + 7 * 4 + 4 + 8
+    assert ctypes.sizeof(_lib.Lut) == 64 and ctypes.sizeof(_lib.Seqs) == 48
+    assert ctypes.sizeof(_lib.FwdArgs) == 4 * 32 + 32 + 64 + 48 + 7 * 4 + 4 + 3 * 8
+    assert ctypes.sizeof(_lib.BwdArgs) == 8 * 32 + 2 * 32 + 8 + 2 * 64 + 48 + 7 * 4 + 4 + 8
 
 
 def test_mask_and_luts_match_fixtures(lut_fixtures):

@@ -1,7 +1,443 @@
-// placeholder until the MFMA backward kernels land
+// MFMA backward kernels for gfx950: bf16 / fp16, head_dim 64 or 128, 64 x 64
+// blocks, equal-length unpadded sequences.  Two passes, no atomics:
+//
+//   dQ pass    (CSR rows)    workgroup = 64 q rows x one q head, 2 waves of 32
+//              rows.  Per listed K/V block: S^T = K Q^T, dP^T = V dO^T (lane =
+//              q row, registers = keys, so lse / delta are per-lane scalars),
+//              dS^T = P^T (dP^T - delta), dQ^T += K^T dS^T with dS^T fed from
+//              registers as the B operand and K^T from LDS transpose reads.
+//   dK/dV pass (CSC columns) workgroup = 64 keys x one kv head (the q heads of
+//              a GQA group are looped inside), 4 waves = 2 key halves x 2 q-row
+//              halves.  K and V fragments stay in registers; per listed q
+//              block: S = Q K^T, dP = dO V^T (lane = key, registers = q rows),
+//              dV^T += dO^T P, dK^T += Q^T dS with P / dS from registers and
+//              dO^T / Q^T from LDS transpose reads.  The two q-row halves are
+//              summed through LDS at the end.
+//
+// Tiles in LDS are row-major with an XOR swizzle of the 16-byte chunks that is
+// conflict-free both for 16-byte row reads (16 lanes on 16 consecutive rows)
+// and for transpose reads (4 rows x 64 bytes per half-wave).
 #include "common.h"
 #include "device_common.h"
+#include "mfma_common.h"
+
 namespace dk {
-bool mfma_bwd_supported(const BwdParams &, int) { return false; }
-int launch_mfma_bwd(const BwdParams &, int, hipStream_t) { return fail(DK_ERR_UNSUPPORTED, "not built"); }
+
+template <int D>
+struct Tile {  // 64 rows x D 16-bit elements, swizzled
+  static constexpr int kRowBytes = D * 2;
+  static constexpr int kBytes = 64 * kRowBytes;
+  static __device__ __forceinline__ int swz(int row) {
+    if constexpr (D == 128)
+      return ((row & 3) << 2) | ((row >> 2) & 3);
+    else
+      return (((row >> 1) & 1) << 2) | ((row >> 2) & 3);
+  }
+  // byte offset of 16-byte chunk `chunk` of `row`
+  static __device__ __forceinline__ int off(int row, int chunk) {
+    return row * kRowBytes + ((chunk ^ swz(row)) << 4);
+  }
+};
+
+// Operand of the transposed tile: lane (d = 32*dt + lane%32, k-group g) gets
+// rows row0 + {4g..4g+3, 8+4g..8+4g+3} of column d.
+template <typename V, int D>
+__device__ __forceinline__ V read_transposed(const char *tile, int row0, int dt, int lane) {
+  const int i16 = lane & 15, dgrp = (lane >> 4) & 1, g = lane >> 5;
+  const int r0 = row0 + 4 * g + (i16 >> 2);
+  const int chunk = 4 * dt + 2 * dgrp + ((i16 & 3) >> 1);
+  const int sub = (i16 & 1) * 8;
+  return lds_read_tr8<V>(tile + Tile<D>::off(r0, chunk) + sub, tile + Tile<D>::off(r0 + 8, chunk) + sub);
+}
+
+// ---------------------------------------------------------------------------
+// dQ pass
+// ---------------------------------------------------------------------------
+template <typename T, int D>
+__global__ __launch_bounds__(128) void mfma_dq_kernel(const BwdParams p, int tiles_y) {
+  using M = Mma<T>;
+  using vec8 = typename M::vec8;
+  using TL = Tile<D>;
+  constexpr int NT = 128;
+  constexpr int KS = D / 16, DT = D / 32, CPR = D / 8;
+  constexpr int CHUNKS = 64 * CPR / NT;
+  constexpr int STAGE = 2 * TL::kBytes;
+  extern __shared__ __align__(16) char smem[];
+
+  const SeqInfo sq = load_seq(p.seqs, blockIdx.z, p.causal);
+  const int tile = tiles_y - 1 - (int)blockIdx.y;
+  if (tile >= seq_row_blocks(sq, 64)) return;
+  const int rb = sq.past / 64 + tile;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int h = blockIdx.x;
+  const int kvh = h / (p.Hq / p.Hkv);
+  const int m = lane & 31, g = lane >> 5;
+  const int row0 = rb * 64 + wave * 32;
+  const int pos = row0 + m;
+  const int qi = pos - sq.past;
+  const bool row_ok = qi >= 0 && qi < sq.q_len;
+
+  vec8 qf[KS], dof[KS];
+  float lse2 = INFINITY, delta = 0.f;
+  {
+    const T *qp = (const T *)p.q.ptr + sq.b * p.q.sb + h * p.q.sh + (int64_t)qi * p.q.st;
+    const T *dop = (const T *)p.dout.ptr + sq.b * p.dout.sb + h * p.dout.sh + (int64_t)qi * p.dout.st;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      uint4 a = make_uint4(0, 0, 0, 0), b = a;
+      if (row_ok) {
+        a = *reinterpret_cast<const uint4 *>(qp + ks * 16 + g * 8);
+        b = *reinterpret_cast<const uint4 *>(dop + ks * 16 + g * 8);
+      }
+      qf[ks] = as_vec8<vec8>(a);
+      dof[ks] = as_vec8<vec8>(b);
+    }
+    if (row_ok) {
+      const float l = p.lse.ptr[sq.b * p.lse.sb + h * p.lse.sh + (int64_t)qi * p.lse.st];
+      lse2 = l == -INFINITY ? INFINITY : l * kLog2e;
+      delta = p.delta[((int64_t)sq.b * p.Hq + h) * p.seqs.max_q_len + qi];
+    }
+  }
+
+  const int lh = lut_head(p.csr, h, p.Hq, p.Hkv);
+  int e0 = 0, e1 = 0;
+  if (rb < p.csr.num_rows) {
+    e0 = p.csr.ptr[lh * p.csr.ptr_sh + rb];
+    e1 = p.csr.ptr[lh * p.csr.ptr_sh + rb + 1];
+  }
+  const int32_t *cols = p.csr.idx + lh * p.csr.idx_sh;
+  const T *kbase = (const T *)p.k.ptr + sq.b * p.k.sb + kvh * p.k.sh;
+  const T *vbase = (const T *)p.v.ptr + sq.b * p.v.sb + kvh * p.v.sh;
+
+  uint4 kreg[CHUNKS], vreg[CHUNKS];
+  auto prefetch = [&](int e) {
+    const int col = cols[e];
+    const int key0 = col * 64;
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+      const int idx = tid + c * NT;
+      const int r = idx / CPR, ch = idx % CPR;
+      kreg[c] = vreg[c] = make_uint4(0, 0, 0, 0);
+      if (col >= 0 && key0 + r < sq.k_len) {
+        kreg[c] = *reinterpret_cast<const uint4 *>(kbase + (int64_t)(key0 + r) * p.k.st + ch * 8);
+        vreg[c] = *reinterpret_cast<const uint4 *>(vbase + (int64_t)(key0 + r) * p.v.st + ch * 8);
+      }
+    }
+  };
+  auto commit = [&](int stage) {
+    char *ks = smem + stage * STAGE, *vs = ks + TL::kBytes;
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+      const int idx = tid + c * NT;
+      const int r = idx / CPR, ch = idx % CPR;
+      *reinterpret_cast<uint4 *>(ks + TL::off(r, ch)) = kreg[c];
+      *reinterpret_cast<uint4 *>(vs + TL::off(r, ch)) = vreg[c];
+    }
+  };
+
+  floatx16 acc[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[dt][r] = 0.f;
+
+  if (e0 < e1) prefetch(e0);
+  for (int e = e0; e < e1; ++e) {
+    const int stage = (e - e0) & 1;
+    const int col = cols[e];
+    commit(stage);
+    __syncthreads();
+    if (e + 1 < e1) prefetch(e + 1);
+    const int key0 = col * 64;
+    if (col < 0 || key0 >= sq.k_len || (p.causal && key0 > row0 + 31)) continue;
+    const char *ks_ = smem + stage * STAGE, *vs_ = ks_ + TL::kBytes;
+
+    floatx16 s[2], dp[2];
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[nt][r] = dp[nt][r] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const vec8 ka = lds_read8<vec8>(ks_ + TL::off(nt * 32 + m, 2 * ks + g));
+        s[nt] = M::mma(ka, qf[ks], s[nt]);
+        const vec8 va = lds_read8<vec8>(vs_ + TL::off(nt * 32 + m, 2 * ks + g));
+        dp[nt] = M::mma(va, dof[ks], dp[nt]);
+      }
+    }
+    const bool need_mask = (key0 + 63 >= sq.k_len) || (p.causal && key0 + 63 > row0);
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        float pr = fast_exp2(s[nt][r] * p.scale_log2 - lse2);
+        if (need_mask) {
+          const int key = key0 + nt * 32 + (r >> 2) * 8 + g * 4 + (r & 3);
+          if (key >= sq.k_len || (p.causal && key > pos)) pr = 0.f;
+        }
+        s[nt][r] = pr * (dp[nt][r] - delta);  // dS^T without sm_scale (applied once at the end)
+      }
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        float f[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) f[i] = s[nt][t * 8 + i];
+        const vec8 dsb = M::pack(f);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          const vec8 kt = read_transposed<vec8, D>(ks_, nt * 32 + t * 16, dt, lane);
+          acc[dt] = M::mma(kt, dsb, acc[dt]);
+        }
+      }
+  }
+
+  if (!row_ok) return;
+  T *dqp = (T *)p.dq.ptr + sq.b * p.dq.sb + h * p.dq.sh + (int64_t)qi * p.dq.st;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int r4 = 0; r4 < 4; ++r4) {
+      T o4[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o4[i] = from_float<T>(acc[dt][r4 * 4 + i] * p.sm_scale);
+      *reinterpret_cast<uint2 *>(dqp + dt * 32 + r4 * 8 + g * 4) = *reinterpret_cast<const uint2 *>(o4);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// dK / dV pass
+// ---------------------------------------------------------------------------
+template <typename T, int D>
+__global__ __launch_bounds__(256) void mfma_dkdv_kernel(const BwdParams p) {
+  using M = Mma<T>;
+  using vec8 = typename M::vec8;
+  using TL = Tile<D>;
+  constexpr int NT = 256;
+  constexpr int KS = D / 16, DT = D / 32, CPR = D / 8;
+  constexpr int CHUNKS = 64 * CPR / NT;
+  constexpr int STAGE = 2 * TL::kBytes + 512;  // Q tile, dO tile, lse2[64], delta[64]
+  extern __shared__ __align__(16) char smem[];
+
+  const SeqInfo sq = load_seq(p.seqs, blockIdx.z, p.causal);
+  const int cb = blockIdx.y;
+  if (cb * 64 >= sq.k_len) return;
+  const int kvh = blockIdx.x;
+  const int ratio = p.Hq / p.Hkv;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int nh = wave & 1, mh = wave >> 1;
+  const int n = lane & 31, g = lane >> 5;
+  const int key = cb * 64 + nh * 32 + n;
+  const bool key_ok = key < sq.k_len;
+
+  vec8 kf[KS], vf[KS];
+  {
+    const T *kp = (const T *)p.k.ptr + sq.b * p.k.sb + kvh * p.k.sh + (int64_t)key * p.k.st;
+    const T *vp = (const T *)p.v.ptr + sq.b * p.v.sb + kvh * p.v.sh + (int64_t)key * p.v.st;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      uint4 a = make_uint4(0, 0, 0, 0), b = a;
+      if (key_ok) {
+        a = *reinterpret_cast<const uint4 *>(kp + ks * 16 + g * 8);
+        b = *reinterpret_cast<const uint4 *>(vp + ks * 16 + g * 8);
+      }
+      kf[ks] = as_vec8<vec8>(a);
+      vf[ks] = as_vec8<vec8>(b);
+    }
+  }
+  floatx16 dk[DT], dv[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) dk[dt][r] = dv[dt][r] = 0.f;
+
+  uint4 qreg[CHUNKS], doreg[CHUNKS];
+  float lreg = 0.f;  // threads 0..63: lse2 of row tid, threads 64..127: delta of row tid-64
+
+  for (int gq = 0; gq < ratio; ++gq) {
+    const int h = kvh * ratio + gq;
+    const int lh = lut_head(p.csc, h, p.Hq, p.Hkv);
+    int e0 = 0, e1 = 0;
+    if (cb < p.csc.num_rows) {
+      e0 = p.csc.ptr[lh * p.csc.ptr_sh + cb];
+      e1 = p.csc.ptr[lh * p.csc.ptr_sh + cb + 1];
+    }
+    const int32_t *rows = p.csc.idx + lh * p.csc.idx_sh;
+    const T *qbase = (const T *)p.q.ptr + sq.b * p.q.sb + h * p.q.sh;
+    const T *dobase = (const T *)p.dout.ptr + sq.b * p.dout.sb + h * p.dout.sh;
+    const float *lsebase = p.lse.ptr + sq.b * p.lse.sb + h * p.lse.sh;
+    const float *deltabase = p.delta + ((int64_t)sq.b * p.Hq + h) * p.seqs.max_q_len;
+
+    auto prefetch = [&](int e) {
+      const int rbq = rows[e];
+      const int pos0 = rbq * 64;
+#pragma unroll
+      for (int c = 0; c < CHUNKS; ++c) {
+        const int idx = tid + c * NT;
+        const int r = idx / CPR, ch = idx % CPR;
+        const int qi = pos0 + r - sq.past;
+        qreg[c] = doreg[c] = make_uint4(0, 0, 0, 0);
+        if (rbq >= 0 && qi >= 0 && qi < sq.q_len) {
+          qreg[c] = *reinterpret_cast<const uint4 *>(qbase + (int64_t)qi * p.q.st + ch * 8);
+          doreg[c] = *reinterpret_cast<const uint4 *>(dobase + (int64_t)qi * p.dout.st + ch * 8);
+        }
+      }
+      if (tid < 128) {
+        const int qi = pos0 + (tid & 63) - sq.past;
+        const bool ok = rbq >= 0 && qi >= 0 && qi < sq.q_len;
+        if (tid < 64) {
+          const float l = ok ? lsebase[(int64_t)qi * p.lse.st] : -INFINITY;
+          lreg = l == -INFINITY ? INFINITY : l * kLog2e;
+        } else {
+          lreg = ok ? deltabase[qi] : 0.f;
+        }
+      }
+    };
+    auto commit = [&](int stage) {
+      char *qs = smem + stage * STAGE, *dos = qs + TL::kBytes;
+#pragma unroll
+      for (int c = 0; c < CHUNKS; ++c) {
+        const int idx = tid + c * NT;
+        const int r = idx / CPR, ch = idx % CPR;
+        *reinterpret_cast<uint4 *>(qs + TL::off(r, ch)) = qreg[c];
+        *reinterpret_cast<uint4 *>(dos + TL::off(r, ch)) = doreg[c];
+      }
+      if (tid < 128) reinterpret_cast<float *>(qs + 2 * TL::kBytes)[tid] = lreg;
+    };
+
+    if (e0 < e1) prefetch(e0);
+    for (int e = e0; e < e1; ++e) {
+      const int stage = (e - e0) & 1;
+      const int rbq = rows[e];
+      commit(stage);
+      __syncthreads();
+      if (e + 1 < e1) prefetch(e + 1);
+      const int pos0 = rbq * 64 + mh * 32;  // first q position of this wave's half
+      if (rbq < 0 || pos0 >= sq.past + sq.q_len || pos0 + 32 <= sq.past) continue;
+      if (p.causal && pos0 + 31 < cb * 64 + nh * 32) continue;  // every row above every key of this wave
+      const char *qs_ = smem + stage * STAGE, *dos_ = qs_ + TL::kBytes;
+      const float *lse_s = reinterpret_cast<const float *>(qs_ + 2 * TL::kBytes);
+      const float *delta_s = lse_s + 64;
+
+      // S = Q K^T, dP = dO V^T : rows = 32 q positions, cols = 32 keys
+      floatx16 s, dp;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[r] = dp[r] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const vec8 qa = lds_read8<vec8>(qs_ + TL::off(mh * 32 + n, 2 * ks + g));
+        s = M::mma(qa, kf[ks], s);
+        const vec8 da = lds_read8<vec8>(dos_ + TL::off(mh * 32 + n, 2 * ks + g));
+        dp = M::mma(da, vf[ks], dp);
+      }
+      const bool need_mask = p.causal && (cb * 64 + nh * 32 + 31 > pos0);
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) {
+        // registers 4*r4 .. +3 are q rows mh*32 + 8*r4 + 4g + {0..3}
+        const float4 l4 = *reinterpret_cast<const float4 *>(lse_s + mh * 32 + r4 * 8 + g * 4);
+        const float4 d4 = *reinterpret_cast<const float4 *>(delta_s + mh * 32 + r4 * 8 + g * 4);
+        const float lv[4] = {l4.x, l4.y, l4.z, l4.w}, dl[4] = {d4.x, d4.y, d4.z, d4.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int r = r4 * 4 + i;
+          float pr = fast_exp2(s[r] * p.scale_log2 - lv[i]);
+          if (need_mask && key > pos0 + r4 * 8 + g * 4 + i) pr = 0.f;
+          if (!key_ok) pr = 0.f;
+          s[r] = pr;                       // P
+          dp[r] = pr * (dp[r] - dl[i]);    // dS without sm_scale
+        }
+      }
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        float pf[8], df[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          pf[i] = s[t * 8 + i];
+          df[i] = dp[t * 8 + i];
+        }
+        const vec8 pb = M::pack(pf), dsb = M::pack(df);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          const vec8 dot = read_transposed<vec8, D>(dos_, mh * 32 + t * 16, dt, lane);
+          dv[dt] = M::mma(dot, pb, dv[dt]);
+          const vec8 qt = read_transposed<vec8, D>(qs_, mh * 32 + t * 16, dt, lane);
+          dk[dt] = M::mma(qt, dsb, dk[dt]);
+        }
+      }
+    }
+    __syncthreads();  // every wave is done with both stages before the next head reuses them
+  }
+
+  // sum the two q-row halves: waves with mh = 1 hand their partials to mh = 0
+  float *red = reinterpret_cast<float *>(smem);
+  if (mh == 1) {
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        red[((nh * 2 + 0) * DT * 16 + dt * 16 + r) * 64 + lane] = dk[dt][r];
+        red[((nh * 2 + 1) * DT * 16 + dt * 16 + r) * 64 + lane] = dv[dt][r];
+      }
+  }
+  __syncthreads();
+  if (mh == 1 || !key_ok) return;
+  T *dkp = (T *)p.dk.ptr + sq.b * p.dk.sb + kvh * p.dk.sh + (int64_t)key * p.dk.st;
+  T *dvp = (T *)p.dv.ptr + sq.b * p.dv.sb + kvh * p.dv.sh + (int64_t)key * p.dv.st;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int r4 = 0; r4 < 4; ++r4) {
+      T k4[4], v4[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int r = r4 * 4 + i;
+        const float a = dk[dt][r] + red[((nh * 2 + 0) * DT * 16 + dt * 16 + r) * 64 + lane];
+        const float b = dv[dt][r] + red[((nh * 2 + 1) * DT * 16 + dt * 16 + r) * 64 + lane];
+        k4[i] = from_float<T>(a * p.sm_scale);
+        v4[i] = from_float<T>(b);
+      }
+      *reinterpret_cast<uint2 *>(dkp + dt * 32 + r4 * 8 + g * 4) = *reinterpret_cast<const uint2 *>(k4);
+      *reinterpret_cast<uint2 *>(dvp + dt * 32 + r4 * 8 + g * 4) = *reinterpret_cast<const uint2 *>(v4);
+    }
+}
+
+bool mfma_bwd_supported(const BwdParams &p, int dtype) {
+  return (dtype == DK_BF16 || dtype == DK_F16) && (p.D == 128 || p.D == 64) && p.csr.block_rows == 64 &&
+         p.csr.block_cols == 64 && p.csr.entry_width == 1 && p.csc.block_rows == 64 && p.csc.block_cols == 64 &&
+         p.vec_ok;
+}
+
+template <typename T, int D>
+static int launch_bwd_td(const BwdParams &p, hipStream_t stream) {
+  const SeqView &s = p.seqs;
+  constexpr int smem_dq = 2 * 2 * Tile<D>::kBytes;
+  constexpr int smem_dkdv_stage = 2 * (2 * Tile<D>::kBytes + 512);
+  constexpr int smem_red = 2 * 2 * (D / 32) * 16 * 64 * 4;
+  constexpr int smem_dkdv = smem_dkdv_stage > smem_red ? smem_dkdv_stage : smem_red;
+  static bool attr_set = false;
+  if (!attr_set) {
+    DK_HIP_CHECK(hipFuncSetAttribute((const void *)mfma_dq_kernel<T, D>,
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, smem_dq));
+    DK_HIP_CHECK(hipFuncSetAttribute((const void *)mfma_dkdv_kernel<T, D>,
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, smem_dkdv));
+    attr_set = true;
+  }
+  const int past = p.causal ? s.max_k_len - s.max_q_len : 0;
+  const int tiles = (past + s.max_q_len - 1) / 64 - past / 64 + 1;
+  const int cblocks = cdiv(s.max_k_len, 64);
+  DK_REQUIRE(tiles <= 65535 && cblocks <= 65535, "sequence too long for one launch");
+  hipLaunchKernelGGL((mfma_dkdv_kernel<T, D>), dim3(p.Hkv, cblocks, s.batch), dim3(256), smem_dkdv, stream, p);
+  DK_HIP_CHECK(hipGetLastError());
+  hipLaunchKernelGGL((mfma_dq_kernel<T, D>), dim3(p.Hq, tiles, s.batch), dim3(128), smem_dq, stream, p, tiles);
+  DK_HIP_CHECK(hipGetLastError());
+  return DK_OK;
+}
+
+int launch_mfma_bwd(const BwdParams &p, int dtype, hipStream_t stream) {
+  if (dtype == DK_BF16)
+    return p.D == 128 ? launch_bwd_td<bf16_t, 128>(p, stream) : launch_bwd_td<bf16_t, 64>(p, stream);
+  return p.D == 128 ? launch_bwd_td<f16_t, 128>(p, stream) : launch_bwd_td<f16_t, 64>(p, stream);
+}
+
 }  // namespace dk

@@ -5,88 +5,113 @@
 // byte is read exactly once, for all q heads of the group together), so the
 // design goal is bytes in flight, not FLOPs:
 //
-//   workgroup = (sequence, kv head, split); its 4 waves each own whole K/V
-//               blocks of the row (round-robin), so 4 x 32 KB of loads are in
-//               flight per workgroup with no barrier between them;
-//   wave      = loads its block with coalesced 16-byte accesses into a private
-//               LDS tile, computes S^T = K Q^T (the q heads of the group are
-//               the MFMA columns), softmax, O^T += V^T P^T with LDS transpose
-//               reads, keeping a private running (max, sum, O);
-//   epilogue  = the 4 waves are merged through LDS into one fp32 partial
-//               (O unnormalised, max, sum) per (sequence, q head, split) in
-//               the caller's workspace; a second small kernel merges the
-//               splits, normalises and writes O and LSE.
+//   work unit = one wave = at most `unit` consecutive entries of the row of
+//               (sequence, kv head); the number of units of a row follows from
+//               its length on the device, so every wave streams the same
+//               amount of K/V whatever the sequence lengths are (workgroups
+//               beyond a row's unit count exit at once);
+//   wave      = per block: computes S^T = K Q^T (the q heads of the group are the MFMA
+//               columns), softmax, O^T += V^T P^T with LDS transpose reads,
+//               keeping a running (max, sum, O) in registers;
+//   epilogue  = one fp32 partial (O unnormalised, max, sum) per (sequence,
+//               q head, unit) in the caller's workspace; a second small
+//               kernel merges the units, normalises and writes O and LSE.
+// A wave works on half blocks (32 keys): 2 x 8.5 KB of private LDS tiles and
+// the next half block prefetched into registers, so 8 waves are resident per
+// CU (2 per SIMD, <= 256 VGPRs each): one wave's loads overlap the other's
+// multiplies on the same SIMD.
+#include <cstdlib>
+
 #include "common.h"
 #include "device_common.h"
 #include "mfma_common.h"
 
 namespace dk {
 
-constexpr int kDecodeSplits = 4;
-constexpr int kDecodeWaves = 4;
+// Blocks per work unit (one wave).  Equal-sized units keep every wave busy for
+// the same time whatever the KV lengths are; 6 blocks = 192 KB per unit.
+static int decode_unit_blocks() {
+  if (const char *env = getenv("DKERNEL_DECODE_UNIT")) {
+    const int v = atoi(env);
+    if (v >= 1 && v <= 64) return v;
+  }
+  return 6;
+}
 
 template <int D>
-struct DecSmem {
-  static constexpr int kKStride = D * 2 + 16;
-  static constexpr int kVStride = D * 2 + 64;
-  static constexpr int kKBytes = 64 * kKStride;
-  static constexpr int kVBytes = 64 * kVStride;
-  static constexpr int kWave = kKBytes + kVBytes;
+struct DecSmem {  // per wave: one 32-key half block of K and of V, plus q of the group
+  static constexpr int kStride = D * 2 + 16;   // bytes per row
+  static constexpr int kHalf = 32 * kStride;   // one half-block tile
+  static constexpr int kQBytes = 32 * D * 2;   // q of up to 32 heads, row-major
+  static constexpr int kWave = 2 * kHalf + kQBytes;
 };
 
-// workspace layout: [batch][Hq][splits][D + 2] floats (O[D], max, sum)
+// workspace layout: [batch][Hq][max_units][D + 2] floats (O[D] unnormalised, max, sum)
 template <typename T, int D>
-__global__ __launch_bounds__(64 * kDecodeWaves) void decode_partial_kernel(const FwdParams p, float *ws) {
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void decode_partial_kernel(const FwdParams p, float *ws, int unit_blocks,
+                                                            int max_units) {
   using M = Mma<T>;
   using vec8 = typename M::vec8;
   using S = DecSmem<D>;
   constexpr int KS = D / 16, DT = D / 32, CPR = D / 8;
-  constexpr int CHUNKS = 64 * CPR / 64;  // 16-byte chunks per lane per tile
   extern __shared__ __align__(16) char smem[];
 
-  const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+  const int unit = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
   const SeqInfo sq = load_seq(p.seqs, b, p.causal);
+  if (sq.q_len <= 0 || sq.k_len <= 0) return;
   const int ratio = p.Hq / p.Hkv;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int lane = threadIdx.x;
   const int m = lane & 31, g = lane >> 5;  // m = q head inside the group (MFMA column)
-  const bool active = sq.q_len > 0 && sq.k_len > 0;
   const int pos = sq.past;                 // absolute position of the single query token
   const int rb = pos / 64;
   const int h0 = kvh * ratio;
+  const int lh = lut_head(p.csr, h0, p.Hq, p.Hkv);
+  if (rb >= p.csr.num_rows) return;
+  const int row0 = p.csr.ptr[lh * p.csr.ptr_sh + rb];
+  const int row1 = p.csr.ptr[lh * p.csr.ptr_sh + rb + 1];
+  const int e0 = row0 + unit * unit_blocks;
+  if (e0 >= row1) return;  // this row has fewer units
+  const int e1 = min(e0 + unit_blocks, row1);
 
-  vec8 qf[KS];
+  // q of the group's heads -> LDS (row min(m, ratio-1) feeds MFMA column m;
+  // columns >= ratio are duplicates whose results are never stored)
+  char *ks_ = smem, *vs_ = smem + S::kHalf, *qs_ = smem + 2 * S::kHalf;
   {
-    const T *qp = (const T *)p.q.ptr + sq.b * p.q.sb + (int64_t)(h0 + m) * p.q.sh + (int64_t)sq.q_start * p.q.st;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      uint4 w = make_uint4(0, 0, 0, 0);
-      if (active && m < ratio) w = *reinterpret_cast<const uint4 *>(qp + ks * 16 + g * 8);
-      qf[ks] = as_vec8<vec8>(w);
+    const int hh = lane / CPR, ch = lane % CPR;  // 64 lanes cover 64 / CPR heads per pass
+    for (int h = hh; h < ratio; h += 64 / CPR) {
+      const T *qp = (const T *)p.q.ptr + sq.b * p.q.sb + (int64_t)(h0 + h) * p.q.sh + (int64_t)sq.q_start * p.q.st;
+      *reinterpret_cast<uint4 *>(qs_ + h * D * 2 + ch * 16) = *reinterpret_cast<const uint4 *>(qp + ch * 8);
     }
   }
-  const int lh = lut_head(p.csr, h0, p.Hq, p.Hkv);
-  int e0 = 0, e1 = 0;
-  if (active && rb < p.csr.num_rows) {
-    e0 = p.csr.ptr[lh * p.csr.ptr_sh + rb];
-    e1 = p.csr.ptr[lh * p.csr.ptr_sh + rb + 1];
-  }
+  const int q_read = (m < ratio ? m : ratio - 1) * D * 2 + g * 16;
   const int32_t *cols = p.csr.idx + lh * p.csr.idx_sh;
   const T *kbase = (const T *)p.k.ptr + sq.b * p.k.sb + kvh * p.k.sh + (int64_t)sq.k_start * p.k.st;
   const T *vbase = (const T *)p.v.ptr + sq.b * p.v.sb + kvh * p.v.sh + (int64_t)sq.k_start * p.v.st;
 
-  char *ks_ = smem + wave * S::kWave, *vs_ = ks_ + S::kKBytes;
-  uint4 kreg[CHUNKS], vreg[CHUNKS];
-  auto prefetch = [&](int e) {
-    const int col = cols[e];
-    const int key0 = col * 64;
+  // half block hb of this unit = keys cols[e0 + hb/2] * 64 + 32 * (hb & 1) + [0, 32)
+  constexpr int HCH = 32 * CPR / 64;  // 16-byte chunks per lane per half tile
+  uint4 kreg[HCH], vreg[HCH];
+  auto prefetch = [&](int hb) {
+    const int col = cols[e0 + (hb >> 1)];
+    const int key0 = col * 64 + (hb & 1) * 32;
+    if (col >= 0 && key0 + 32 <= sq.k_len) {  // whole half inside the sequence: no per-row guards
 #pragma unroll
-    for (int c = 0; c < CHUNKS; ++c) {
-      const int idx = lane + c * 64;
-      const int r = idx / CPR, ch = idx % CPR;
-      kreg[c] = vreg[c] = make_uint4(0, 0, 0, 0);
-      if (col >= 0 && key0 + r < sq.k_len) {
+      for (int c = 0; c < HCH; ++c) {
+        const int idx = lane + c * 64;
+        const int r = idx / CPR, ch = idx % CPR;
         kreg[c] = *reinterpret_cast<const uint4 *>(kbase + (int64_t)(key0 + r) * p.k.st + ch * 8);
         vreg[c] = *reinterpret_cast<const uint4 *>(vbase + (int64_t)(key0 + r) * p.v.st + ch * 8);
+      }
+    } else {
+#pragma unroll
+      for (int c = 0; c < HCH; ++c) {
+        const int idx = lane + c * 64;
+        const int r = idx / CPR, ch = idx % CPR;
+        kreg[c] = vreg[c] = make_uint4(0, 0, 0, 0);
+        if (col >= 0 && key0 + r < sq.k_len) {
+          kreg[c] = *reinterpret_cast<const uint4 *>(kbase + (int64_t)(key0 + r) * p.k.st + ch * 8);
+          vreg[c] = *reinterpret_cast<const uint4 *>(vbase + (int64_t)(key0 + r) * p.v.st + ch * 8);
+        }
       }
     }
   };
@@ -98,69 +123,67 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void decode_partial_kernel(const
     for (int r = 0; r < 16; ++r) oacc[dt][r] = 0.f;
   float m_run = -INFINITY, l_run = 0.f;
 
-  const int k_read = m * S::kKStride + g * 16;
+  const int k_read = m * S::kStride + g * 16;
   const int i16 = lane & 15, dgrp = (lane >> 4) & 1;
-  const int v_read = (4 * g + (i16 >> 2)) * S::kVStride + (16 * dgrp + 4 * (i16 & 3)) * 2;
-  constexpr int STEP = kDecodeSplits * kDecodeWaves;
+  const int v_read = (4 * g + (i16 >> 2)) * S::kStride + (16 * dgrp + 4 * (i16 & 3)) * 2;
+  const int nhalf = 2 * (e1 - e0);
 
-  int e = e0 + split * kDecodeWaves + wave;
-  if (e < e1) prefetch(e);
-  for (; e < e1; e += STEP) {
-    const int col = cols[e];
-    const int key0 = col * 64;
-    // this wave's private tile: the previous block's reads are complete
-    // (program order within the wave), so it can be overwritten
+  prefetch(0);
+  for (int hb = 0; hb < nhalf; ++hb) {
+    const int col = cols[e0 + (hb >> 1)];
+    const int key0 = col * 64 + (hb & 1) * 32;
+    // The tiles are private to this wave and LDS operations of one wave
+    // execute in order, so the previous half block's reads are done; only the
+    // compiler must not reorder across these points (a memory fence would
+    // also drain the global prefetch issued next).
+    asm volatile("" ::: "memory");
 #pragma unroll
-    for (int c = 0; c < CHUNKS; ++c) {
+    for (int c = 0; c < HCH; ++c) {
       const int idx = lane + c * 64;
       const int r = idx / CPR, ch = idx % CPR;
-      *reinterpret_cast<uint4 *>(ks_ + r * S::kKStride + ch * 16) = kreg[c];
-      *reinterpret_cast<uint4 *>(vs_ + r * S::kVStride + ch * 16) = vreg[c];
+      *reinterpret_cast<uint4 *>(ks_ + r * S::kStride + ch * 16) = kreg[c];
+      *reinterpret_cast<uint4 *>(vs_ + r * S::kStride + ch * 16) = vreg[c];
     }
-    if (e + STEP < e1) prefetch(e + STEP);
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    asm volatile("" ::: "memory");
+    if (hb + 1 < nhalf) prefetch(hb + 1);
     if (col < 0 || key0 >= sq.k_len || (p.causal && key0 > pos)) continue;
 
-    floatx16 sacc[2];
+    floatx16 sacc;
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) sacc[nt][r] = 0.f;
+    for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
+    {
+      vec8 a[KS], qb[KS];
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
-        vec8 a = lds_read8<vec8>(ks_ + k_read + nt * 32 * S::kKStride + ks * 32);
-        sacc[nt] = M::mma(a, qf[ks], sacc[nt]);
+        a[ks] = lds_read8<vec8>(ks_ + k_read + ks * 32);
+        qb[ks] = lds_read8<vec8>(qs_ + q_read + ks * 32);
       }
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) sacc = M::mma(a[ks], qb[ks], sacc);
     }
-    const bool need_mask = (key0 + 63 >= sq.k_len) || (p.causal && key0 + 63 > pos);
+    const bool need_mask = (key0 + 31 >= sq.k_len) || (p.causal && key0 + 31 > pos);
     float mx = -INFINITY;
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        float s = sacc[nt][r] * p.scale_log2;
-        if (need_mask) {
-          const int key = key0 + nt * 32 + (r >> 2) * 8 + g * 4 + (r & 3);
-          if (key >= sq.k_len || (p.causal && key > pos)) s = -INFINITY;
-        }
-        sacc[nt][r] = s;
-        mx = fmaxf(mx, s);
+    for (int r = 0; r < 16; ++r) {
+      float sv = sacc[r] * p.scale_log2;
+      if (need_mask) {
+        const int key = key0 + (r >> 2) * 8 + g * 4 + (r & 3);
+        if (key >= sq.k_len || (p.causal && key > pos)) sv = -INFINITY;
       }
+      sacc[r] = sv;
+      mx = fmaxf(mx, sv);
+    }
     mx = fmaxf(mx, xor32(mx));
     const float m_new = fmaxf(m_run, mx);
     const float m_use = m_new == -INFINITY ? 0.f : m_new;
     const float alpha = fast_exp2(m_run - m_use);
     float psum = 0.f;
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const float pv = fast_exp2(sacc[nt][r] - m_use);
-        sacc[nt][r] = pv;
-        psum += pv;
-      }
+    for (int r = 0; r < 16; ++r) {
+      const float pv = fast_exp2(sacc[r] - m_use);
+      sacc[r] = pv;
+      psum += pv;
+    }
     psum += xor32(psum);
     l_run = l_run * alpha + psum;
     m_run = m_new;
@@ -169,76 +192,55 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void decode_partial_kernel(const
 #pragma unroll
       for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt)
+    for (int t = 0; t < 2; ++t) {
+      float pf[8];
 #pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        float pf[8];
+      for (int i = 0; i < 8; ++i) pf[i] = sacc[t * 8 + i];
+      const vec8 pb = M::pack(pf);
+      const char *vrow = vs_ + v_read + t * 16 * S::kStride;
+      vec8 a[DT];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) pf[i] = sacc[nt][t * 8 + i];
-        const vec8 pb = M::pack(pf);
-        const char *vrow = vs_ + v_read + (nt * 32 + t * 16) * S::kVStride;
+      for (int dt = 0; dt < DT; ++dt) a[dt] = lds_read_tr8<vec8>(vrow + dt * 64, vrow + 8 * S::kStride + dt * 64);
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-          vec8 a = lds_read_tr8<vec8>(vrow + dt * 64, vrow + 8 * S::kVStride + dt * 64);
-          oacc[dt] = M::mma(a, pb, oacc[dt]);
-        }
-      }
+      for (int dt = 0; dt < DT; ++dt) oacc[dt] = M::mma(a[dt], pb, oacc[dt]);
+    }
   }
 
-  // ---- merge the 4 waves through LDS (tiles are dead now) ----
-  __syncthreads();
-  float *red_o = reinterpret_cast<float *>(smem);            // [wave][head][D]
-  float *red_ml = red_o + kDecodeWaves * 32 * D;             // [wave][head][2]
+  // ---- partial result of this unit: lanes (m < ratio) hold head h0 + m ----
   if (m < ratio) {
+    float *dst = ws + (((int64_t)b * p.Hq + h0 + m) * max_units + unit) * (D + 2);
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-      for (int r = 0; r < 16; ++r)
-        red_o[(wave * 32 + m) * D + dt * 32 + (r >> 2) * 8 + g * 4 + (r & 3)] = oacc[dt][r];
+      for (int r4 = 0; r4 < 4; ++r4)
+        *reinterpret_cast<float4 *>(dst + dt * 32 + r4 * 8 + g * 4) =
+            make_float4(oacc[dt][r4 * 4], oacc[dt][r4 * 4 + 1], oacc[dt][r4 * 4 + 2], oacc[dt][r4 * 4 + 3]);
     if (g == 0) {
-      red_ml[(wave * 32 + m) * 2 + 0] = m_run;
-      red_ml[(wave * 32 + m) * 2 + 1] = l_run;
-    }
-  }
-  __syncthreads();
-  for (int idx = tid; idx < ratio * D; idx += 64 * kDecodeWaves) {
-    const int hh = idx / D, d = idx % D;
-    float mw[kDecodeWaves], mmax = -INFINITY;
-#pragma unroll
-    for (int w = 0; w < kDecodeWaves; ++w) {
-      mw[w] = red_ml[(w * 32 + hh) * 2];
-      mmax = fmaxf(mmax, mw[w]);
-    }
-    const float muse = mmax == -INFINITY ? 0.f : mmax;
-    float o = 0.f, l = 0.f;
-#pragma unroll
-    for (int w = 0; w < kDecodeWaves; ++w) {
-      const float sc = fast_exp2(mw[w] - muse);
-      o += sc * red_o[(w * 32 + hh) * D + d];
-      l += sc * red_ml[(w * 32 + hh) * 2 + 1];
-    }
-    float *dst = ws + (((int64_t)b * p.Hq + h0 + hh) * kDecodeSplits + split) * (D + 2);
-    dst[d] = o;
-    if (d == 0) {
-      dst[D] = mmax;
-      dst[D + 1] = l;
+      dst[D] = m_run;
+      dst[D + 1] = l_run;
     }
   }
 }
 
 template <typename T, int D>
-__global__ __launch_bounds__(D) void decode_combine_kernel(const FwdParams p, const float *ws) {
+__global__ __launch_bounds__(D) void decode_combine_kernel(const FwdParams p, const float *ws, int unit_blocks,
+                                                           int max_units) {
   const int h = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
   const SeqInfo sq = load_seq(p.seqs, b, p.causal);
   if (sq.q_len <= 0) return;
-  const float *src = ws + ((int64_t)b * p.Hq + h) * kDecodeSplits * (D + 2);
+  int units = 0;
+  const int rb = sq.past / 64;
+  if (sq.k_len > 0 && rb < p.csr.num_rows) {
+    const int lh = lut_head(p.csr, h, p.Hq, p.Hkv);
+    const int n = p.csr.ptr[lh * p.csr.ptr_sh + rb + 1] - p.csr.ptr[lh * p.csr.ptr_sh + rb];
+    units = (n + unit_blocks - 1) / unit_blocks;
+  }
+  const float *src = ws + ((int64_t)b * p.Hq + h) * max_units * (D + 2);
   float mmax = -INFINITY;
-#pragma unroll
-  for (int s = 0; s < kDecodeSplits; ++s) mmax = fmaxf(mmax, src[s * (D + 2) + D]);
+  for (int s = 0; s < units; ++s) mmax = fmaxf(mmax, src[s * (D + 2) + D]);
   const float muse = mmax == -INFINITY ? 0.f : mmax;
   float o = 0.f, l = 0.f;
-#pragma unroll
-  for (int s = 0; s < kDecodeSplits; ++s) {
+  for (int s = 0; s < units; ++s) {
     const float sc = fast_exp2(src[s * (D + 2) + D] - muse);
     o += sc * src[s * (D + 2) + d];
     l += sc * src[s * (D + 2) + D + 1];
@@ -251,6 +253,13 @@ __global__ __launch_bounds__(D) void decode_combine_kernel(const FwdParams p, co
         l > 0.f ? (mmax + log2f(l)) * kLn2 : -INFINITY;
 }
 
+// Upper bound on the entries of one table row: the caller's hint when given,
+// else the number of column blocks.
+static int decode_max_row_entries(const FwdParams &p) {
+  return p.csr.max_row_entries > 0 ? p.csr.max_row_entries : p.csr.num_rows;
+}
+static int decode_max_units(const FwdParams &p) { return cdiv(decode_max_row_entries(p), decode_unit_blocks()); }
+
 bool decode_supported(const FwdParams &p, int dtype) {
   const int ratio = p.Hq / p.Hkv;
   const bool shared_row = p.csr.num_heads == 1 || (p.csr.num_heads == p.Hkv && p.Hkv != p.Hq) || ratio == 1 ||
@@ -261,24 +270,19 @@ bool decode_supported(const FwdParams &p, int dtype) {
 }
 
 size_t decode_workspace_bytes(const FwdParams &p) {
-  return (size_t)p.seqs.batch * p.Hq * kDecodeSplits * (p.D + 2) * sizeof(float);
+  return (size_t)p.seqs.batch * p.Hq * decode_max_units(p) * (p.D + 2) * sizeof(float);
 }
 
 template <typename T, int D>
 static int launch_decode_td(const FwdParams &p, float *ws, hipStream_t stream) {
-  constexpr int tiles = kDecodeWaves * DecSmem<D>::kWave;
-  constexpr int red = (kDecodeWaves * 32 * D + kDecodeWaves * 32 * 2) * 4;
-  constexpr int smem = tiles > red ? tiles : red;
-  static bool attr_set = false;
-  if (!attr_set) {
-    DK_HIP_CHECK(hipFuncSetAttribute((const void *)decode_partial_kernel<T, D>,
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, smem));
-    attr_set = true;
-  }
-  hipLaunchKernelGGL((decode_partial_kernel<T, D>), dim3(kDecodeSplits, p.Hkv, p.seqs.batch),
-                     dim3(64 * kDecodeWaves), smem, stream, p, ws);
+  constexpr int smem = DecSmem<D>::kWave;
+  const int unit_blocks = decode_unit_blocks(), max_units = decode_max_units(p);
+  DK_REQUIRE(max_units <= 65535, "too many decode units");
+  hipLaunchKernelGGL((decode_partial_kernel<T, D>), dim3(max_units, p.Hkv, p.seqs.batch), dim3(64), smem, stream,
+                     p, ws, unit_blocks, max_units);
   DK_HIP_CHECK(hipGetLastError());
-  hipLaunchKernelGGL((decode_combine_kernel<T, D>), dim3(p.Hq, p.seqs.batch), dim3(D), 0, stream, p, ws);
+  hipLaunchKernelGGL((decode_combine_kernel<T, D>), dim3(p.Hq, p.seqs.batch), dim3(D), 0, stream, p, ws,
+                     unit_blocks, max_units);
   DK_HIP_CHECK(hipGetLastError());
   return DK_OK;
 }

@@ -87,15 +87,24 @@ __global__ __launch_bounds__(128 * G) void mfma_fwd_kernel(const FwdParams p, in
   auto prefetch = [&](int e) {
     const int col = cols[e];
     const int key0 = col * 64;
+    if (col >= 0 && key0 + 64 <= sq.k_len) {  // whole block inside the sequence: no per-row guards
 #pragma unroll
-    for (int c = 0; c < CHUNKS; ++c) {
-      const int idx = tid + c * NT;
-      const int r = idx / CPR, ch = idx % CPR;
-      const bool ok = col >= 0 && key0 + r < sq.k_len;
-      kreg[c] = vreg[c] = make_uint4(0, 0, 0, 0);
-      if (ok) {
+      for (int c = 0; c < CHUNKS; ++c) {
+        const int idx = tid + c * NT;
+        const int r = idx / CPR, ch = idx % CPR;
         kreg[c] = *reinterpret_cast<const uint4 *>(kbase + (int64_t)(key0 + r) * p.k.st + ch * 8);
         vreg[c] = *reinterpret_cast<const uint4 *>(vbase + (int64_t)(key0 + r) * p.v.st + ch * 8);
+      }
+    } else {
+#pragma unroll
+      for (int c = 0; c < CHUNKS; ++c) {
+        const int idx = tid + c * NT;
+        const int r = idx / CPR, ch = idx % CPR;
+        kreg[c] = vreg[c] = make_uint4(0, 0, 0, 0);
+        if (col >= 0 && key0 + r < sq.k_len) {
+          kreg[c] = *reinterpret_cast<const uint4 *>(kbase + (int64_t)(key0 + r) * p.k.st + ch * 8);
+          vreg[c] = *reinterpret_cast<const uint4 *>(vbase + (int64_t)(key0 + r) * p.v.st + ch * 8);
+        }
       }
     }
   };
@@ -133,72 +142,93 @@ __global__ __launch_bounds__(128 * G) void mfma_fwd_kernel(const FwdParams p, in
     if (col < 0 || key0 >= sq.k_len || (p.causal && key0 > row0 + 31)) continue;  // nothing visible (wave-uniform)
     const char *ks_ = smem + stage * S::kStage, *vs_ = ks_ + S::kKBytes;
 
-    // S^T = K Q^T : two 32-key tiles
+    // S^T = K Q^T : two 32-key tiles.  Operand reads run one tile ahead of the
+    // multiplies so that LDS latency is hidden behind the MFMA pipe.
     floatx16 sacc[2];
-#pragma unroll
-    for (int nt = 0; nt < 2; ++nt) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) sacc[nt][r] = 0.f;
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        vec8 a = lds_read8<vec8>(ks_ + k_read + nt * 32 * S::kKStride + ks * 32);
-        sacc[nt] = M::mma(a, qf[ks], sacc[nt]);
-      }
-    }
-
-    // scale, mask, online softmax.  Register r of tile nt is key 32nt + 8(r/4) + 4g + r%4.
-    const bool need_mask = (key0 + 63 >= sq.k_len) || (p.causal && key0 + 63 > row0);
-    float mx = -INFINITY;
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        float s = sacc[nt][r] * p.scale_log2;
-        if (need_mask) {
-          const int key = key0 + nt * 32 + (r >> 2) * 8 + g * 4 + (r & 3);
-          if (key >= sq.k_len || (p.causal && key > pos)) s = -INFINITY;
-        }
-        sacc[nt][r] = s;
-        mx = fmaxf(mx, s);
+      for (int r = 0; r < 16; ++r) sacc[nt][r] = 0.f;
+    {
+      vec8 ka[KS];
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) ka[ks] = lds_read8<vec8>(ks_ + k_read + ks * 32);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        sacc[0] = M::mma(ka[ks], qf[ks], sacc[0]);
+        ka[ks] = lds_read8<vec8>(ks_ + k_read + 32 * S::kKStride + ks * 32);
       }
-    mx = fmaxf(mx, xor32(mx));
-    const float m_new = fmaxf(m_run, mx);
-    const float m_use = m_new == -INFINITY ? 0.f : m_new;
-    const float alpha = fast_exp2(m_run - m_use);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) sacc[1] = M::mma(ka[ks], qf[ks], sacc[1]);
+    }
+    // first V^T operands do not depend on the softmax: fetch them now
+    vec8 va[2][DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+      va[0][dt] = lds_read_tr8<vec8>(vs_ + v_read + dt * 64, vs_ + v_read + 8 * S::kVStride + dt * 64);
+
+    // online softmax in the log2 domain.  Register r of tile nt is key
+    // 32nt + 8(r/4) + 4g + r%4.  m_run is a reference maximum that is only
+    // raised when a row's maximum grows by more than 2^8 (the accumulator
+    // and the row sum stay consistent with it, so the result is exact).
+    const bool need_mask = (key0 + 63 >= sq.k_len) || (p.causal && key0 + 63 > row0);
+    if (need_mask) {
+      const int lim = p.causal ? min(pos, sq.k_len - 1) : sq.k_len - 1;  // last visible key of this row
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int key = key0 + nt * 32 + (r >> 2) * 8 + g * 4 + (r & 3);
+          sacc[nt][r] = key > lim ? -INFINITY : sacc[nt][r];
+        }
+    }
+    float mx = fmaxf(sacc[0][0], sacc[1][0]);
+#pragma unroll
+    for (int r = 1; r < 16; ++r) mx = fmaxf(mx, fmaxf(sacc[0][r], sacc[1][r]));
+    mx = fmaxf(mx, xor32(mx)) * p.scale_log2;  // scale > 0: max commutes with it
+    if (__builtin_amdgcn_ballot_w64(mx > m_run + 8.f) != 0) {  // wave-uniform: some row needs a new reference
+      const float m_new = fmaxf(m_run, mx);
+      const float alpha = fast_exp2(m_run - (m_new == -INFINITY ? 0.f : m_new));
+      l_run *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
+      m_run = m_new;
+    }
+    const float m_use = m_run == -INFINITY ? 0.f : m_run;
     float psum = 0.f;
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const float pv = fast_exp2(sacc[nt][r] - m_use);
+        const float pv = fast_exp2(fmaf(sacc[nt][r], p.scale_log2, -m_use));
         sacc[nt][r] = pv;
         psum += pv;
       }
-    psum += xor32(psum);
-    l_run = l_run * alpha + psum;
-    m_run = m_new;
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
+    l_run += psum;  // per-lane partial row sum; the two half-waves are added once in the epilogue
 
     // O^T += V^T P^T : k-step (nt, t) covers keys 32nt + 16t + {4g..4g+3, 8+4g..8+4g+3}
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt)
+    for (int step = 0; step < 4; ++step) {
+      const int nt = step >> 1, t = step & 1;
+      float pf[8];
 #pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        float pf[8];
+      for (int i = 0; i < 8; ++i) pf[i] = sacc[nt][t * 8 + i];
+      const vec8 pb = M::pack(pf);
+      if (step < 3) {
+        const char *vrow = vs_ + v_read + ((step + 1) * 16) * S::kVStride;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) pf[i] = sacc[nt][t * 8 + i];
-        const vec8 pb = M::pack(pf);
-        const char *vrow = vs_ + v_read + (nt * 32 + t * 16) * S::kVStride;
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-          vec8 a = lds_read_tr8<vec8>(vrow + dt * 64, vrow + 8 * S::kVStride + dt * 64);
-          oacc[dt] = M::mma(a, pb, oacc[dt]);
-        }
+        for (int dt = 0; dt < DT; ++dt)
+          va[(step + 1) & 1][dt] = lds_read_tr8<vec8>(vrow + dt * 64, vrow + 8 * S::kVStride + dt * 64);
       }
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) oacc[dt] = M::mma(va[step & 1][dt], pb, oacc[dt]);
+    }
   }
+
+  // l_run holds this lane's share of the row sum (keys with this lane's g)
+  l_run += xor32(l_run);
 
   // ---- epilogue: O = O^T / l, LSE = (m + log2 l) ln 2 ----
   if (!row_ok) return;

@@ -118,6 +118,11 @@ class SparseAttention(torch.nn.Module):
             layout_csr = [zero_stride(x) for x in layout_csr]
             layout_csc = [zero_stride(x) for x in layout_csc]
 
+        # longest row of the table: sizes the split-KV decode grid
+        crow = layout_csr[0]
+        self.lut_max_row = int((crow[:, 1:] - crow[:, :-1]).max()) if crow.size(1) > 1 else 0
+        self.kwargs['lut_max_row'] = self.lut_max_row
+
         self.register_buffer("layout_csr_crow", layout_csr[0].to(torch.int32), persistent=False)
         self.register_buffer("layout_csr_col", layout_csr[1].to(torch.int32), persistent=False)
         self.register_buffer("layout_csc_ccol", layout_csc[0].to(torch.int32), persistent=False)

@@ -62,7 +62,7 @@ def _rowvec(x: Optional[Tensor], strides=None) -> _lib.RowVec:
     return _lib.RowVec(x.data_ptr(), sb, sh, st)
 
 
-def _lut(layout: Tuple[Tensor, Tensor, int, int], device, group: int = 1) -> _lib.Lut:
+def _lut(layout: Tuple[Tensor, Tensor, int, int], device, group: int = 1, max_row: int = 0) -> _lib.Lut:
     ptr, idx, block_rows, block_cols = layout
     assert ptr.dtype == torch.int32 and idx.dtype == torch.int32
     assert ptr.device == device and idx.device == device, \
@@ -77,7 +77,22 @@ def _lut(layout: Tuple[Tensor, Tensor, int, int], device, group: int = 1) -> _li
     else:
         assert idx.stride(-1) == 1 or idx.size(-1) <= 1
     return _lib.Lut(ptr.data_ptr(), idx.data_ptr(), ptr.stride(0), idx.stride(0), width,
-                    ptr.size(0), ptr.size(1) - 1, int(block_rows), int(block_cols), int(group))
+                    ptr.size(0), ptr.size(1) - 1, int(block_rows), int(block_cols), int(group), int(max_row))
+
+
+_CONST_I32 = {}
+
+
+def _const_i32(device, n: int, value: int) -> Tensor:
+    """Cached constant int32 vector (sequence starts / ends that do not depend
+    on the data), so that a decode step launches no fill kernels."""
+    key = (device, n, value)
+    t = _CONST_I32.get(key)
+    if t is None:
+        if len(_CONST_I32) > 64:
+            _CONST_I32.clear()
+        t = _CONST_I32[key] = torch.full((n,), value, dtype=torch.int32, device=device)
+    return t
 
 
 def _stream() -> C.c_void_p:
@@ -104,7 +119,8 @@ def _forward(ctx, q: Tensor, k: Tensor, v: Tensor, sm_scale: float,
              return_lse: bool = False,
              causal=True,
              split_qkv=None,
-             lut_group: int = 1) -> Tuple[Tensor, Optional[Tensor]]:
+             lut_group: int = 1,
+             lut_max_row: int = 0) -> Tuple[Tensor, Optional[Tensor]]:
     """Unpadded 4-D forward (training, prefill, single-token decode).
     Reference: dkernel/ops/sparse_attn_fwd.py:383-567.  `d_splits` is accepted
     and ignored (a Triton shared-memory workaround)."""
@@ -130,7 +146,7 @@ def _forward(ctx, q: Tensor, k: Tensor, v: Tensor, sm_scale: float,
     args = _lib.FwdArgs()
     args.q, args.k, args.v, args.o = (_tensor4(x, hdim, seq_dim) for x in (q, k, v, o))
     args.lse = _rowvec(lse)
-    args.csr = _lut(layout_csr, q.device, lut_group)
+    args.csr = _lut(layout_csr, q.device, lut_group, lut_max_row)
     args.seqs = _lib.Seqs(q.size(0), qlen, klen, 0, None, None, None, None)
     args.num_q_heads, args.num_kv_heads, args.head_dim = num_heads, num_kv_heads, q.size(-1)
     args.dtype, args.causal, args.impl = _DTYPES[q.dtype], int(bool(causal)), _impl
@@ -199,7 +215,8 @@ def padded_sparse_attn(q: Tensor, k: Tensor, v: Tensor, sm_scale: float,
                        inference: bool = True,
                        causal: bool = True,
                        return_lse: bool = False,
-                       lut_group: int = 1):
+                       lut_group: int = 1,
+                       lut_max_row: int = 0):
     """4-D inputs with left paddings and / or explicit sequence lengths; q has
     either one token per sequence (decode) or the same padded length as k.
     Reference: dkernel/ops/sparse_attn_inference.py:10-147.  Padding rows of
@@ -220,22 +237,23 @@ def padded_sparse_attn(q: Tensor, k: Tensor, v: Tensor, sm_scale: float,
         assert k_len <= max_seqlen, \
             f'k has seqlen {k_len} while max sequence length is set to {max_seqlen}.'
     q, k, v = _unit_last(q), _unit_last(k), _unit_last(v)
-    out = out if out is not None else q.new_zeros(q.shape)
-
     dev = q.device
+    if out is None:
+        # decode writes every row; padded prefill leaves the padding rows untouched, so they start at zero
+        out = q.new_empty(q.shape) if q_len == 1 else q.new_zeros(q.shape)
+
     if left_paddings is not None:
         assert left_paddings.shape == (batches,)
         k_starts = left_paddings.to(dev, dtype=torch.int32).contiguous()
     else:
-        k_starts = torch.zeros((batches,), dtype=torch.int32, device=dev)
+        k_starts = _const_i32(dev, batches, 0)
     if seqlens is not None:
         # ends beyond the padded length are clamped on the device
         k_ends = k_starts + seqlens.to(dev, dtype=torch.int32)
     else:
-        k_ends = torch.full_like(k_starts, k_len)
+        k_ends = _const_i32(dev, batches, k_len)
     if q_len == 1:
-        q_starts = torch.zeros_like(k_starts)
-        q_ends = q_starts + 1
+        q_starts, q_ends = _const_i32(dev, batches, 0), _const_i32(dev, batches, 1)
     else:
         q_starts, q_ends = k_starts, k_ends
 
@@ -245,7 +263,7 @@ def padded_sparse_attn(q: Tensor, k: Tensor, v: Tensor, sm_scale: float,
     args = _lib.FwdArgs()
     args.q, args.k, args.v, args.o = (_tensor4(x, hdim, seq_dim) for x in (q, k, v, out))
     args.lse = _rowvec(lse)
-    args.csr = _lut(sparse_layout, dev, lut_group)
+    args.csr = _lut(sparse_layout, dev, lut_group, lut_max_row)
     args.seqs = _lib.Seqs(batches, q_len, k_len, 0, q_starts.data_ptr(), q_ends.data_ptr(),
                           k_starts.data_ptr(), k_ends.data_ptr())
     args.num_q_heads, args.num_kv_heads, args.head_dim = num_heads, num_kv_heads, head_size
@@ -382,14 +400,15 @@ class _sparse_attention(torch.autograd.Function):
                 ctx.message = "Currently does not support paddings in inputs. WIP."
                 res = padded_sparse_attn(q, k, v, sm_scale, layout_csr, left_paddings=left_paddings,
                                          seqlens=seqlens, seq_dim=seq_dim, max_seqlen=max_seqlen,
-                                         causal=causal, return_lse=return_lse, lut_group=lut_group)
+                                         causal=causal, return_lse=return_lse, lut_group=lut_group,
+                                         lut_max_row=kwargs.get("lut_max_row", 0))
                 output, lse = res if return_lse else (res, None)
             else:
                 ctx.support_backward = True
                 ctx.message = ""
                 fwd_kwargs = {k_: v_ for k_, v_ in kwargs.items()
                               if k_ in ("inference", "out", "d_splits", "max_seqlen", "return_lse",
-                                        "causal", "split_qkv", "lut_group")}
+                                        "causal", "split_qkv", "lut_group", "lut_max_row")}
                 output, lse = _forward(ctx, q, k, v, sm_scale, layout_csr, seq_dim=seq_dim, **fwd_kwargs)
         return output, lse
 

@@ -108,6 +108,8 @@ typedef struct dk_lut {
   int32_t block_cols;  /* tokens per listed entry */
   int32_t group;       /* consecutive table heads known to hold identical rows (1 if unknown);
                           lets heads of a GQA group share K/V tiles inside a workgroup */
+  int32_t max_row_entries; /* largest number of entries in one row (0 if unknown); sizes the
+                              split-KV decode grid and workspace */
 } dk_lut;
 
 /* Sequence geometry.  With all four pointers NULL every sequence has

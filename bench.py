@@ -101,6 +101,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip backward / decode figures")
     ap.add_argument("--impl", default="auto", choices=["auto", "generic", "mfma"])
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="run a plain 1 GiB device copy and exit (scale for the FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the path has no cross-GPU component in this build "
@@ -109,6 +111,14 @@ def main():
         sys.exit(2)
 
     import torch
+    if args.calibrate_copy:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda:0").fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_bytes_read": 1 << 30, "copy_bytes_written": 1 << 30, "copies": 3}))
+        return
     from dkernel_amd import LocalStrideSparseAttention, ops
     ops.set_impl(args.impl)
     dev = "cuda:0"

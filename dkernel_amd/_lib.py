@@ -9,7 +9,8 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libdkernel_hip.so")
+# DKERNEL_AMD_LIB points at another build of the same library (A/B comparisons of kernel variants)
+LIB_PATH = os.environ.get("DKERNEL_AMD_LIB") or os.path.join(_HERE, "libdkernel_hip.so")
 
 DK_BF16, DK_F16, DK_F32 = 0, 1, 2
 DK_IMPL_AUTO, DK_IMPL_GENERIC, DK_IMPL_MFMA = 0, 1, 2

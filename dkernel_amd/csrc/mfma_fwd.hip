@@ -19,6 +19,8 @@
 // Grid: x = head group (fastest, so that the 8 XCDs, which receive
 // workgroups round-robin, each keep a fixed set of kv heads in their L2),
 // y = q tile with the longest rows first, z = batch.
+#include <cstdlib>
+
 #include "common.h"
 #include "device_common.h"
 #include "mfma_common.h"
@@ -35,7 +37,7 @@ struct FwdSmem {
 };
 
 template <typename T, int D, int G>
-__global__ __launch_bounds__(128 * G) void mfma_fwd_kernel(const FwdParams p, int tiles_y) {
+__global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(2, 2))) void mfma_fwd_kernel(const FwdParams p, int tiles_y) {
   using M = Mma<T>;
   using vec8 = typename M::vec8;
   using S = FwdSmem<D>;
@@ -149,23 +151,28 @@ __global__ __launch_bounds__(128 * G) void mfma_fwd_kernel(const FwdParams p, in
     for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
       for (int r = 0; r < 16; ++r) sacc[nt][r] = 0.f;
-    {
-      vec8 ka[KS];
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) ka[ks] = lds_read8<vec8>(ks_ + k_read + ks * 32);
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        sacc[0] = M::mma(ka[ks], qf[ks], sacc[0]);
-        ka[ks] = lds_read8<vec8>(ks_ + k_read + 32 * S::kKStride + ks * 32);
-      }
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) sacc[1] = M::mma(ka[ks], qf[ks], sacc[1]);
-    }
-    // first V^T operands do not depend on the softmax: fetch them now
+    // The scheduler barriers pin the order "issue a batch of LDS reads, then
+    // multiply the previous batch": left alone, the compiler sinks every read
+    // next to its MFMA and each multiply then waits out the LDS latency.
     vec8 va[2][DT];
+    {
+      vec8 ka[2][KS];
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-      va[0][dt] = lds_read_tr8<vec8>(vs_ + v_read + dt * 64, vs_ + v_read + 8 * S::kVStride + dt * 64);
+      for (int ks = 0; ks < KS; ++ks) ka[0][ks] = lds_read8<vec8>(ks_ + k_read + ks * 32);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) ka[1][ks] = lds_read8<vec8>(ks_ + k_read + 32 * S::kKStride + ks * 32);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) sacc[0] = M::mma(ka[0][ks], qf[ks], sacc[0]);
+      // first V^T operands do not depend on the softmax: fetch them behind the multiplies
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+        va[0][dt] = lds_read_tr8<vec8>(vs_ + v_read + dt * 64, vs_ + v_read + 8 * S::kVStride + dt * 64);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) sacc[1] = M::mma(ka[1][ks], qf[ks], sacc[1]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
 
     // online softmax in the log2 domain.  Register r of tile nt is key
     // 32nt + 8(r/4) + 4g + r%4.  m_run is a reference maximum that is only
@@ -206,7 +213,9 @@ __global__ __launch_bounds__(128 * G) void mfma_fwd_kernel(const FwdParams p, in
         sacc[nt][r] = pv;
         psum += pv;
       }
-    l_run += psum;  // per-lane partial row sum; the two half-waves are added once in the epilogue
+    // fp32 sum of the unrounded probabilities (the LSE has to hold 1e-3); per-lane partial,
+    // the two half-waves are added once in the epilogue
+    l_run += psum;
 
     // O^T += V^T P^T : k-step (nt, t) covers keys 32nt + 16t + {4g..4g+3, 8+4g..8+4g+3}
 #pragma unroll
@@ -254,10 +263,11 @@ __global__ __launch_bounds__(128 * G) void mfma_fwd_kernel(const FwdParams p, in
 // the look-up-table row.
 static int fwd_group(const FwdParams &p) {
   const int ratio = p.Hq / p.Hkv;
+  static const int max_group = getenv("DKERNEL_FWD_GROUP") ? atoi(getenv("DKERNEL_FWD_GROUP")) : 4;
   // a table with one row per q head may differ inside a kv group
   const int same_lut = (p.csr.num_heads == p.Hq && p.Hq != p.Hkv) ? p.csr.group : ratio;
   for (int g = 4; g > 1; g >>= 1)
-    if (ratio % g == 0 && same_lut % g == 0) return g;
+    if (g <= max_group && ratio % g == 0 && same_lut % g == 0) return g;
   return 1;
 }
 

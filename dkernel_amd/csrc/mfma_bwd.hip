@@ -1,8 +1,9 @@
 // MFMA backward kernels for gfx950: bf16 / fp16, head_dim 64 or 128, 64 x 64
 // blocks, equal-length unpadded sequences.  Two passes, no atomics:
 //
-//   dQ pass    (CSR rows)    workgroup = 64 q rows x one q head, 2 waves of 32
-//              rows.  Per listed K/V block: S^T = K Q^T, dP^T = V dO^T (lane =
+//   dQ pass    (CSR rows)    workgroup = 64 q rows x one q head, 4 waves = 2 row
+//              halves x 2 key halves (2 waves per SIMD; the key halves are
+//              summed through LDS at the end).  Per listed K/V block: S^T = K Q^T, dP^T = V dO^T (lane =
 //              q row, registers = keys, so lse / delta are per-lane scalars),
 //              dS^T = P^T (dP^T - delta), dQ^T += K^T dS^T with dS^T fed from
 //              registers as the B operand and K^T from LDS transpose reads.
@@ -14,53 +15,25 @@
 //              dO^T / Q^T from LDS transpose reads.  The two q-row halves are
 //              summed through LDS at the end.
 //
-// Tiles in LDS are row-major with an XOR swizzle of the 16-byte chunks that is
-// conflict-free both for 16-byte row reads (16 lanes on 16 consecutive rows)
-// and for transpose reads (4 rows x 64 bytes per half-wave).
+// Tiles are copied HBM -> LDS asynchronously (no staging registers), double
+// buffered, in the swizzled row-major layout of mfma_common.h.
 #include "common.h"
 #include "device_common.h"
 #include "mfma_common.h"
 
 namespace dk {
 
-template <int D>
-struct Tile {  // 64 rows x D 16-bit elements, swizzled
-  static constexpr int kRowBytes = D * 2;
-  static constexpr int kBytes = 64 * kRowBytes;
-  static __device__ __forceinline__ int swz(int row) {
-    if constexpr (D == 128)
-      return ((row & 3) << 2) | ((row >> 2) & 3);
-    else
-      return (((row >> 1) & 1) << 2) | ((row >> 2) & 3);
-  }
-  // byte offset of 16-byte chunk `chunk` of `row`
-  static __device__ __forceinline__ int off(int row, int chunk) {
-    return row * kRowBytes + ((chunk ^ swz(row)) << 4);
-  }
-};
-
-// Operand of the transposed tile: lane (d = 32*dt + lane%32, k-group g) gets
-// rows row0 + {4g..4g+3, 8+4g..8+4g+3} of column d.
-template <typename V, int D>
-__device__ __forceinline__ V read_transposed(const char *tile, int row0, int dt, int lane) {
-  const int i16 = lane & 15, dgrp = (lane >> 4) & 1, g = lane >> 5;
-  const int r0 = row0 + 4 * g + (i16 >> 2);
-  const int chunk = 4 * dt + 2 * dgrp + ((i16 & 3) >> 1);
-  const int sub = (i16 & 1) * 8;
-  return lds_read_tr8<V>(tile + Tile<D>::off(r0, chunk) + sub, tile + Tile<D>::off(r0 + 8, chunk) + sub);
-}
-
 // ---------------------------------------------------------------------------
 // dQ pass
 // ---------------------------------------------------------------------------
 template <typename T, int D>
-__global__ __launch_bounds__(128) void mfma_dq_kernel(const BwdParams p, int tiles_y) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void mfma_dq_kernel(const BwdParams p,
+                                                                                                   int tiles_y) {
   using M = Mma<T>;
   using vec8 = typename M::vec8;
   using TL = Tile<D>;
-  constexpr int NT = 128;
-  constexpr int KS = D / 16, DT = D / 32, CPR = D / 8;
-  constexpr int CHUNKS = 64 * CPR / NT;
+  constexpr int NT = 256;
+  constexpr int KS = D / 16, DT = D / 32;
   constexpr int STAGE = 2 * TL::kBytes;
   extern __shared__ __align__(16) char smem[];
 
@@ -68,11 +41,13 @@ __global__ __launch_bounds__(128) void mfma_dq_kernel(const BwdParams p, int til
   const int tile = tiles_y - 1 - (int)blockIdx.y;
   if (tile >= seq_row_blocks(sq, 64)) return;
   const int rb = sq.past / 64 + tile;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int rh = wave & 1, kh = wave >> 1;  // q-row half, key half
   const int h = blockIdx.x;
   const int kvh = h / (p.Hq / p.Hkv);
   const int m = lane & 31, g = lane >> 5;
-  const int row0 = rb * 64 + wave * 32;
+  const int row0 = rb * 64 + rh * 32;
   const int pos = row0 + m;
   const int qi = pos - sq.past;
   const bool row_ok = qi >= 0 && qi < sq.q_len;
@@ -109,31 +84,22 @@ __global__ __launch_bounds__(128) void mfma_dq_kernel(const BwdParams p, int til
   const T *kbase = (const T *)p.k.ptr + sq.b * p.k.sb + kvh * p.k.sh;
   const T *vbase = (const T *)p.v.ptr + sq.b * p.v.sb + kvh * p.v.sh;
 
-  uint4 kreg[CHUNKS], vreg[CHUNKS];
-  auto prefetch = [&](int e) {
+  TileLoader<D, NT> kload, vload;
+  kload.init(tid, p.k.st);
+  vload.init(tid, p.v.st);
+  auto issue = [&](int e, int stage) {  // asynchronous copy of block e's K and V tiles into `stage`
     const int col = cols[e];
     const int key0 = col * 64;
-#pragma unroll
-    for (int c = 0; c < CHUNKS; ++c) {
-      const int idx = tid + c * NT;
-      const int r = idx / CPR, ch = idx % CPR;
-      kreg[c] = vreg[c] = make_uint4(0, 0, 0, 0);
-      if (col >= 0 && key0 + r < sq.k_len) {
-        kreg[c] = *reinterpret_cast<const uint4 *>(kbase + (int64_t)(key0 + r) * p.k.st + ch * 8);
-        vreg[c] = *reinterpret_cast<const uint4 *>(vbase + (int64_t)(key0 + r) * p.v.st + ch * 8);
-      }
-    }
+    const int valid = col < 0 ? 0 : sq.k_len - key0;
+    char *ks = smem + stage * STAGE;
+    kload.issue(reinterpret_cast<const char *>(kbase + (int64_t)key0 * p.k.st), 0, valid, ks);
+    vload.issue(reinterpret_cast<const char *>(vbase + (int64_t)key0 * p.v.st), 0, valid, ks + TL::kBytes);
   };
-  auto commit = [&](int stage) {
-    char *ks = smem + stage * STAGE, *vs = ks + TL::kBytes;
+  // operand read offsets inside this wave's key half: row kh*32 + m, chunk 2ks+g swizzled
+  int rd[KS], tr[DT][2];
 #pragma unroll
-    for (int c = 0; c < CHUNKS; ++c) {
-      const int idx = tid + c * NT;
-      const int r = idx / CPR, ch = idx % CPR;
-      *reinterpret_cast<uint4 *>(ks + TL::off(r, ch)) = kreg[c];
-      *reinterpret_cast<uint4 *>(vs + TL::off(r, ch)) = vreg[c];
-    }
-  };
+  for (int ks = 0; ks < KS; ++ks) rd[ks] = TL::off(kh * 32 + m, 2 * ks + g);
+  transposed_offsets<D>(lane, tr);
 
   floatx16 acc[DT];
 #pragma unroll
@@ -141,59 +107,83 @@ __global__ __launch_bounds__(128) void mfma_dq_kernel(const BwdParams p, int til
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[dt][r] = 0.f;
 
-  if (e0 < e1) prefetch(e0);
+  if (e0 < e1) issue(e0, 0);
   for (int e = e0; e < e1; ++e) {
     const int stage = (e - e0) & 1;
     const int col = cols[e];
-    commit(stage);
-    __syncthreads();
-    if (e + 1 < e1) prefetch(e + 1);
-    const int key0 = col * 64;
+    wait_tile_loads();
+    __syncthreads();  // tile e is visible; every wave is done with the other stage
+    if (e + 1 < e1) issue(e + 1, stage ^ 1);
+    const int key0 = col * 64 + kh * 32;  // first key of this wave's half
     if (col < 0 || key0 >= sq.k_len || (p.causal && key0 > row0 + 31)) continue;
     const char *ks_ = smem + stage * STAGE, *vs_ = ks_ + TL::kBytes;
 
-    floatx16 s[2], dp[2];
+    floatx16 s, dp;
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt) {
+    for (int r = 0; r < 16; ++r) s[r] = dp[r] = 0.f;
+    // batches of operand reads, then the multiplies (the scheduler barriers keep
+    // the compiler from sinking each read next to its MFMA)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) s[nt][r] = dp[nt][r] = 0.f;
+    for (int half = 0; half < 2; ++half) {
+      vec8 ka[KS / 2];
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const vec8 ka = lds_read8<vec8>(ks_ + TL::off(nt * 32 + m, 2 * ks + g));
-        s[nt] = M::mma(ka, qf[ks], s[nt]);
-        const vec8 va = lds_read8<vec8>(vs_ + TL::off(nt * 32 + m, 2 * ks + g));
-        dp[nt] = M::mma(va, dof[ks], dp[nt]);
+      for (int i = 0; i < KS / 2; ++i) ka[i] = lds_read8<vec8>(ks_ + rd[half * (KS / 2) + i]);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < KS / 2; ++i) s = M::mma(ka[i], qf[half * (KS / 2) + i], s);
+    }
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      vec8 va[KS / 2];
+#pragma unroll
+      for (int i = 0; i < KS / 2; ++i) va[i] = lds_read8<vec8>(vs_ + rd[half * (KS / 2) + i]);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < KS / 2; ++i) dp = M::mma(va[i], dof[half * (KS / 2) + i], dp);
+    }
+    // K^T operands of the dQ product do not depend on dS: fetch them now
+    const char *krow = ks_ + kh * 32 * TL::kRowBytes;
+    vec8 kt[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) kt[dt] = lds_read_tr8<vec8>(krow + tr[dt][0], krow + tr[dt][1]);
+
+    const bool need_mask = (key0 + 31 >= sq.k_len) || (p.causal && key0 + 31 > row0);
+    const int lim = p.causal ? min(pos, sq.k_len - 1) : sq.k_len - 1;  // last visible key of this row
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      float pr = fast_exp2(fmaf(s[r], p.scale_log2, -lse2));
+      if (need_mask) {
+        const int key = key0 + (r >> 2) * 8 + g * 4 + (r & 3);
+        pr = key > lim ? 0.f : pr;
+      }
+      s[r] = pr * (dp[r] - delta);  // dS^T without sm_scale (applied once at the end)
+    }
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      float f[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) f[i] = s[t * 8 + i];
+      const vec8 dsb = M::pack(f);
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        acc[dt] = M::mma(kt[dt], dsb, acc[dt]);
+        if (t == 0)  // refill with the second k-step's operand as soon as the register is free
+          kt[dt] = lds_read_tr8<vec8>(krow + 16 * TL::kRowBytes + tr[dt][0], krow + 16 * TL::kRowBytes + tr[dt][1]);
       }
     }
-    const bool need_mask = (key0 + 63 >= sq.k_len) || (p.causal && key0 + 63 > row0);
-#pragma unroll
-    for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        float pr = fast_exp2(s[nt][r] * p.scale_log2 - lse2);
-        if (need_mask) {
-          const int key = key0 + nt * 32 + (r >> 2) * 8 + g * 4 + (r & 3);
-          if (key >= sq.k_len || (p.causal && key > pos)) pr = 0.f;
-        }
-        s[nt][r] = pr * (dp[nt][r] - delta);  // dS^T without sm_scale (applied once at the end)
-      }
-#pragma unroll
-    for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        float f[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) f[i] = s[nt][t * 8 + i];
-        const vec8 dsb = M::pack(f);
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-          const vec8 kt = read_transposed<vec8, D>(ks_, nt * 32 + t * 16, dt, lane);
-          acc[dt] = M::mma(kt, dsb, acc[dt]);
-        }
-      }
   }
 
-  if (!row_ok) return;
+  // sum the two key halves: waves with kh = 1 hand their partial to kh = 0
+  __syncthreads();
+  float *red = reinterpret_cast<float *>(smem);
+  if (kh == 1) {
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) red[((rh * DT + dt) * 16 + r) * 64 + lane] = acc[dt][r];
+  }
+  __syncthreads();
+  if (kh == 1 || !row_ok) return;
   T *dqp = (T *)p.dq.ptr + sq.b * p.dq.sb + h * p.dq.sh + (int64_t)qi * p.dq.st;
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt)
@@ -201,7 +191,10 @@ __global__ __launch_bounds__(128) void mfma_dq_kernel(const BwdParams p, int til
     for (int r4 = 0; r4 < 4; ++r4) {
       T o4[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) o4[i] = from_float<T>(acc[dt][r4 * 4 + i] * p.sm_scale);
+      for (int i = 0; i < 4; ++i) {
+        const int r = r4 * 4 + i;
+        o4[i] = from_float<T>((acc[dt][r] + red[((rh * DT + dt) * 16 + r) * 64 + lane]) * p.sm_scale);
+      }
       *reinterpret_cast<uint2 *>(dqp + dt * 32 + r4 * 8 + g * 4) = *reinterpret_cast<const uint2 *>(o4);
     }
 }
@@ -215,8 +208,7 @@ __global__ __launch_bounds__(256) void mfma_dkdv_kernel(const BwdParams p) {
   using vec8 = typename M::vec8;
   using TL = Tile<D>;
   constexpr int NT = 256;
-  constexpr int KS = D / 16, DT = D / 32, CPR = D / 8;
-  constexpr int CHUNKS = 64 * CPR / NT;
+  constexpr int KS = D / 16, DT = D / 32;
   constexpr int STAGE = 2 * TL::kBytes + 512;  // Q tile, dO tile, lse2[64], delta[64]
   extern __shared__ __align__(16) char smem[];
 
@@ -252,8 +244,14 @@ __global__ __launch_bounds__(256) void mfma_dkdv_kernel(const BwdParams p) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) dk[dt][r] = dv[dt][r] = 0.f;
 
-  uint4 qreg[CHUNKS], doreg[CHUNKS];
   float lreg = 0.f;  // threads 0..63: lse2 of row tid, threads 64..127: delta of row tid-64
+  TileLoader<D, NT> qload, doload;
+  qload.init(tid, p.q.st);
+  doload.init(tid, p.dout.st);
+  int rd[KS], tr[DT][2];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) rd[ks] = TL::off(mh * 32 + n, 2 * ks + g);
+  transposed_offsets<D>(lane, tr);
 
   for (int gq = 0; gq < ratio; ++gq) {
     const int h = kvh * ratio + gq;
@@ -269,22 +267,18 @@ __global__ __launch_bounds__(256) void mfma_dkdv_kernel(const BwdParams p) {
     const float *lsebase = p.lse.ptr + sq.b * p.lse.sb + h * p.lse.sh;
     const float *deltabase = p.delta + ((int64_t)sq.b * p.Hq + h) * p.seqs.max_q_len;
 
-    auto prefetch = [&](int e) {
+    // asynchronous copy of q block rows[e] (Q and dO tiles) into `stage`; lse / delta of
+    // its 64 rows are fetched into one register per thread and stored by `commit`
+    auto issue = [&](int e, int stage) {
       const int rbq = rows[e];
-      const int pos0 = rbq * 64;
-#pragma unroll
-      for (int c = 0; c < CHUNKS; ++c) {
-        const int idx = tid + c * NT;
-        const int r = idx / CPR, ch = idx % CPR;
-        const int qi = pos0 + r - sq.past;
-        qreg[c] = doreg[c] = make_uint4(0, 0, 0, 0);
-        if (rbq >= 0 && qi >= 0 && qi < sq.q_len) {
-          qreg[c] = *reinterpret_cast<const uint4 *>(qbase + (int64_t)qi * p.q.st + ch * 8);
-          doreg[c] = *reinterpret_cast<const uint4 *>(dobase + (int64_t)qi * p.dout.st + ch * 8);
-        }
-      }
+      const int qi0 = rbq * 64 - sq.past;  // query index of the tile's first row
+      // rows before the first query (qi < 0, when k is longer than q) and beyond the last are zero-filled
+      const int lo = rbq < 0 ? 64 : -qi0, hi = sq.q_len - qi0;
+      char *qs = smem + stage * STAGE;
+      qload.issue(reinterpret_cast<const char *>(qbase + (int64_t)qi0 * p.q.st), lo, hi, qs);
+      doload.issue(reinterpret_cast<const char *>(dobase + (int64_t)qi0 * p.dout.st), lo, hi, qs + TL::kBytes);
       if (tid < 128) {
-        const int qi = pos0 + (tid & 63) - sq.past;
+        const int qi = qi0 + (tid & 63);
         const bool ok = rbq >= 0 && qi >= 0 && qi < sq.q_len;
         if (tid < 64) {
           const float l = ok ? lsebase[(int64_t)qi * p.lse.st] : -INFINITY;
@@ -295,24 +289,17 @@ __global__ __launch_bounds__(256) void mfma_dkdv_kernel(const BwdParams p) {
       }
     };
     auto commit = [&](int stage) {
-      char *qs = smem + stage * STAGE, *dos = qs + TL::kBytes;
-#pragma unroll
-      for (int c = 0; c < CHUNKS; ++c) {
-        const int idx = tid + c * NT;
-        const int r = idx / CPR, ch = idx % CPR;
-        *reinterpret_cast<uint4 *>(qs + TL::off(r, ch)) = qreg[c];
-        *reinterpret_cast<uint4 *>(dos + TL::off(r, ch)) = doreg[c];
-      }
-      if (tid < 128) reinterpret_cast<float *>(qs + 2 * TL::kBytes)[tid] = lreg;
+      if (tid < 128) reinterpret_cast<float *>(smem + stage * STAGE + 2 * TL::kBytes)[tid] = lreg;
     };
 
-    if (e0 < e1) prefetch(e0);
+    if (e0 < e1) issue(e0, 0);
     for (int e = e0; e < e1; ++e) {
       const int stage = (e - e0) & 1;
       const int rbq = rows[e];
+      wait_tile_loads();
       commit(stage);
-      __syncthreads();
-      if (e + 1 < e1) prefetch(e + 1);
+      __syncthreads();  // tile e is visible; every wave is done with the other stage
+      if (e + 1 < e1) issue(e + 1, stage ^ 1);
       const int pos0 = rbq * 64 + mh * 32;  // first q position of this wave's half
       if (rbq < 0 || pos0 >= sq.past + sq.q_len || pos0 + 32 <= sq.past) continue;
       if (p.causal && pos0 + 31 < cb * 64 + nh * 32) continue;  // every row above every key of this wave
@@ -324,12 +311,19 @@ __global__ __launch_bounds__(256) void mfma_dkdv_kernel(const BwdParams p) {
       floatx16 s, dp;
 #pragma unroll
       for (int r = 0; r < 16; ++r) s[r] = dp[r] = 0.f;
+      {
+        vec8 qa[KS], da[KS];
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const vec8 qa = lds_read8<vec8>(qs_ + TL::off(mh * 32 + n, 2 * ks + g));
-        s = M::mma(qa, kf[ks], s);
-        const vec8 da = lds_read8<vec8>(dos_ + TL::off(mh * 32 + n, 2 * ks + g));
-        dp = M::mma(da, vf[ks], dp);
+        for (int ks = 0; ks < KS; ++ks) {
+          qa[ks] = lds_read8<vec8>(qs_ + rd[ks]);
+          da[ks] = lds_read8<vec8>(dos_ + rd[ks]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          s = M::mma(qa[ks], kf[ks], s);
+          dp = M::mma(da[ks], vf[ks], dp);
+        }
       }
       const bool need_mask = p.causal && (cb * 64 + nh * 32 + 31 > pos0);
 #pragma unroll
@@ -341,9 +335,9 @@ __global__ __launch_bounds__(256) void mfma_dkdv_kernel(const BwdParams p) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int r = r4 * 4 + i;
-          float pr = fast_exp2(s[r] * p.scale_log2 - lv[i]);
-          if (need_mask && key > pos0 + r4 * 8 + g * 4 + i) pr = 0.f;
-          if (!key_ok) pr = 0.f;
+          float pr = fast_exp2(fmaf(s[r], p.scale_log2, -lv[i]));
+          if (need_mask) pr = key > pos0 + r4 * 8 + g * 4 + i ? 0.f : pr;
+          pr = key_ok ? pr : 0.f;
           s[r] = pr;                       // P
           dp[r] = pr * (dp[r] - dl[i]);    // dS without sm_scale
         }
@@ -357,12 +351,17 @@ __global__ __launch_bounds__(256) void mfma_dkdv_kernel(const BwdParams p) {
           df[i] = dp[t * 8 + i];
         }
         const vec8 pb = M::pack(pf), dsb = M::pack(df);
+        const int rowoff = (mh * 32 + t * 16) * TL::kRowBytes;
+        vec8 dot[DT], qt[DT];
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
-          const vec8 dot = read_transposed<vec8, D>(dos_, mh * 32 + t * 16, dt, lane);
-          dv[dt] = M::mma(dot, pb, dv[dt]);
-          const vec8 qt = read_transposed<vec8, D>(qs_, mh * 32 + t * 16, dt, lane);
-          dk[dt] = M::mma(qt, dsb, dk[dt]);
+          dot[dt] = lds_read_tr8<vec8>(dos_ + rowoff + tr[dt][0], dos_ + rowoff + tr[dt][1]);
+          qt[dt] = lds_read_tr8<vec8>(qs_ + rowoff + tr[dt][0], qs_ + rowoff + tr[dt][1]);
+        }
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          dv[dt] = M::mma(dot[dt], pb, dv[dt]);
+          dk[dt] = M::mma(qt[dt], dsb, dk[dt]);
         }
       }
     }
@@ -402,6 +401,17 @@ __global__ __launch_bounds__(256) void mfma_dkdv_kernel(const BwdParams p) {
     }
 }
 
+// Explicit instantiations: with only the implicit ones the fp16 host stubs of
+// these kernels are not emitted by this compiler version.
+template __global__ void mfma_dq_kernel<bf16_t, 128>(const BwdParams, int);
+template __global__ void mfma_dq_kernel<bf16_t, 64>(const BwdParams, int);
+template __global__ void mfma_dq_kernel<f16_t, 128>(const BwdParams, int);
+template __global__ void mfma_dq_kernel<f16_t, 64>(const BwdParams, int);
+template __global__ void mfma_dkdv_kernel<bf16_t, 128>(const BwdParams);
+template __global__ void mfma_dkdv_kernel<bf16_t, 64>(const BwdParams);
+template __global__ void mfma_dkdv_kernel<f16_t, 128>(const BwdParams);
+template __global__ void mfma_dkdv_kernel<f16_t, 64>(const BwdParams);
+
 bool mfma_bwd_supported(const BwdParams &p, int dtype) {
   return (dtype == DK_BF16 || dtype == DK_F16) && (p.D == 128 || p.D == 64) && p.csr.block_rows == 64 &&
          p.csr.block_cols == 64 && p.csr.entry_width == 1 && p.csc.block_rows == 64 && p.csc.block_cols == 64 &&
@@ -429,7 +439,7 @@ static int launch_bwd_td(const BwdParams &p, hipStream_t stream) {
   DK_REQUIRE(tiles <= 65535 && cblocks <= 65535, "sequence too long for one launch");
   hipLaunchKernelGGL((mfma_dkdv_kernel<T, D>), dim3(p.Hkv, cblocks, s.batch), dim3(256), smem_dkdv, stream, p);
   DK_HIP_CHECK(hipGetLastError());
-  hipLaunchKernelGGL((mfma_dq_kernel<T, D>), dim3(p.Hq, tiles, s.batch), dim3(128), smem_dq, stream, p, tiles);
+  hipLaunchKernelGGL((mfma_dq_kernel<T, D>), dim3(p.Hq, tiles, s.batch), dim3(256), smem_dq, stream, p, tiles);
   DK_HIP_CHECK(hipGetLastError());
   return DK_OK;
 }

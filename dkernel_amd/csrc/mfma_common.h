@@ -79,6 +79,99 @@ __device__ __forceinline__ V lds_read_tr8(const char *p0, const char *p1) {
   return __builtin_bit_cast(V, r);
 }
 
+// ---------------------------------------------------------------------------
+// 64-row x D tile of 16-bit elements in LDS, row-major, with an XOR swizzle of
+// the 16-byte chunks that is conflict-free both for 16-byte row reads (16 lanes
+// on 16 consecutive rows) and for transpose reads (4 rows x 64 bytes per
+// half-wave).  The swizzle only depends on row & 15.
+// ---------------------------------------------------------------------------
+template <int D>
+struct Tile {
+  static constexpr int kRowBytes = D * 2;
+  static constexpr int kBytes = 64 * kRowBytes;
+  static constexpr int kChunksPerRow = D / 8;
+  static __device__ __forceinline__ int swz(int row) {
+    if constexpr (D == 128)
+      return ((row & 3) << 2) | ((row >> 2) & 3);
+    else
+      return (((row >> 1) & 1) << 2) | ((row >> 2) & 3);
+  }
+  // byte offset of 16-byte chunk `chunk` of `row`
+  static __device__ __forceinline__ int off(int row, int chunk) {
+    return row * kRowBytes + ((chunk ^ swz(row)) << 4);
+  }
+};
+
+// Per-lane byte offsets of the two transpose reads of d-tile dt, relative to
+// row0 of the tile, for row0 a multiple of 16; loop invariants, so no address
+// arithmetic is left in the inner loops (the row0 part becomes an immediate).
+// The lane (d = 32*dt + lane%32, k-group g) receives rows
+// row0 + {4g..4g+3, 8+4g..8+4g+3} of column d.
+template <int D>
+__device__ __forceinline__ void transposed_offsets(int lane, int (&off)[D / 32][2]) {
+  const int i16 = lane & 15, dgrp = (lane >> 4) & 1, g = lane >> 5;
+  const int r0 = 4 * g + (i16 >> 2);
+#pragma unroll
+  for (int dt = 0; dt < D / 32; ++dt) {
+    const int chunk = 4 * dt + 2 * dgrp + ((i16 & 3) >> 1);
+    off[dt][0] = Tile<D>::off(r0, chunk) + (i16 & 1) * 8;
+    off[dt][1] = Tile<D>::off(r0 + 8, chunk) + (i16 & 1) * 8;
+  }
+}
+
+// Asynchronous global -> LDS copy of one tile by NT threads, straight into LDS
+// (no staging registers, no ds_write): a wave instruction moves 64 x 16 bytes
+// to 1 KB of consecutive LDS; the swizzle is realised by choosing which global
+// chunk each lane fetches (lane position p of row r fetches chunk p ^ swz(r)).
+// TileLoader::init computes the per-thread global byte offsets once.  Rows
+// outside [lo, hi) are zero-filled with ordinary LDS stores.  The caller
+// waits (wait_tile_loads) and synchronises before reading the tile.
+template <int D, int NT>
+struct TileLoader {
+  static constexpr int kCPR = D / 8;
+  static constexpr int kChunks = 64 * kCPR / NT;
+  uint32_t goff[kChunks];  // global byte offset of this thread's chunk c inside the 64-row block
+  int row0;                // first row this thread's wave covers with chunk 0 (wave-uniform)
+  int lane_row, lane_byte;
+
+  __device__ __forceinline__ void init(int tid, int64_t row_stride_elems) {
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    row0 = wave * (64 / kCPR);
+    lane_row = lane / kCPR;
+    lane_byte = lane * 16;
+#pragma unroll
+    for (int c = 0; c < kChunks; ++c) {
+      const int r = row0 + c * (NT / kCPR) + lane_row;
+      const int pos = lane % kCPR;
+      goff[c] = (uint32_t)(r * row_stride_elems) * 2u + (uint32_t)((pos ^ Tile<D>::swz(r)) << 4);
+    }
+  }
+  // rows [lo, hi) of the block are copied, the others zero-filled
+  __device__ __forceinline__ void issue(const char *gblk, int lo, int hi, char *tile) const {
+    typedef __attribute__((address_space(3))) void *lds_ptr;
+    if (lo <= 0 && hi >= 64) {
+#pragma unroll
+      for (int c = 0; c < kChunks; ++c)
+        __builtin_amdgcn_global_load_lds(gblk + goff[c], (lds_ptr)(tile + (row0 + c * (NT / kCPR)) * Tile<D>::kRowBytes),
+                                         16, 0, 0);
+    } else {
+#pragma unroll
+      for (int c = 0; c < kChunks; ++c) {
+        char *wbase = tile + (row0 + c * (NT / kCPR)) * Tile<D>::kRowBytes;
+        const int r = row0 + c * (NT / kCPR) + lane_row;
+        if (r >= lo && r < hi)
+          __builtin_amdgcn_global_load_lds(gblk + goff[c], (lds_ptr)wbase, 16, 0, 0);
+        else
+          *reinterpret_cast<uint4 *>(wbase + lane_byte) = make_uint4(0, 0, 0, 0);
+      }
+    }
+  }
+};
+
+// All asynchronous tile loads (and any other vector memory loads) of this wave have landed.
+__device__ __forceinline__ void wait_tile_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // Exchange with the lane 32 away (the other half-wave that holds the rest of

@@ -37,7 +37,7 @@ struct FwdSmem {
 };
 
 template <typename T, int D, int G>
-__global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(2, 2))) void mfma_fwd_kernel(const FwdParams p, int tiles_y) {
+__global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 ? 1 : 2, 2))) void mfma_fwd_kernel(const FwdParams p, int tiles_y) {
   using M = Mma<T>;
   using vec8 = typename M::vec8;
   using S = FwdSmem<D>;

@@ -13,8 +13,8 @@
 // half-wave, and feeds P^T to the second product O^T += V^T P^T as the B
 // operand straight from registers.  V stays row-major in LDS; its transposed
 // operand comes from LDS transpose reads.  K/V tiles are double buffered in
-// LDS (one barrier per block), the next tile's global loads are in flight
-// while the current one is being multiplied.
+// LDS (one barrier per block) and copied HBM -> LDS asynchronously, without
+// staging registers, while the current one is being multiplied.
 //
 // Grid: x = head group (fastest, so that the 8 XCDs, which receive
 // workgroups round-robin, each keep a fixed set of kv heads in their L2),
@@ -28,12 +28,8 @@
 namespace dk {
 
 template <int D>
-struct FwdSmem {
-  static constexpr int kKStride = D * 2 + 16;  // bytes; 16 rows cover all banks for 16-byte reads
-  static constexpr int kVStride = D * 2 + 64;  // bytes; 4 rows x 64 B cover all banks for transpose reads
-  static constexpr int kKBytes = 64 * kKStride;
-  static constexpr int kVBytes = 64 * kVStride;
-  static constexpr int kStage = kKBytes + kVBytes;
+struct FwdSmem {  // one stage = K tile + V tile, swizzled row-major (mfma_common.h)
+  static constexpr int kStage = 2 * Tile<D>::kBytes;
 };
 
 template <typename T, int D, int G>
@@ -44,8 +40,7 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
   constexpr int NT = 128 * G;   // threads
   constexpr int KS = D / 16;    // k-steps of the QK^T product
   constexpr int DT = D / 32;    // d-tiles of the output
-  constexpr int CPR = D / 8;    // 16-byte chunks per K/V row
-  constexpr int CHUNKS = 64 * CPR / NT;  // chunks per thread per tile
+  using TL = Tile<D>;
   extern __shared__ __align__(16) char smem[];
 
   SeqInfo sq;
@@ -84,41 +79,17 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
   const T *kbase = (const T *)p.k.ptr + sq.b * p.k.sb + kvh * p.k.sh + (int64_t)sq.k_start * p.k.st;
   const T *vbase = (const T *)p.v.ptr + sq.b * p.v.sb + kvh * p.v.sh + (int64_t)sq.k_start * p.v.st;
 
-  // ---- global -> register prefetch of one K/V tile ----
-  uint4 kreg[CHUNKS], vreg[CHUNKS];
-  auto prefetch = [&](int e) {
+  // ---- asynchronous HBM -> LDS copy of one K/V tile pair (no staging registers) ----
+  TileLoader<D, NT> kload, vload;
+  kload.init(tid, p.k.st);
+  vload.init(tid, p.v.st);
+  auto issue = [&](int e, int stage) {
     const int col = cols[e];
     const int key0 = col * 64;
-    if (col >= 0 && key0 + 64 <= sq.k_len) {  // whole block inside the sequence: no per-row guards
-#pragma unroll
-      for (int c = 0; c < CHUNKS; ++c) {
-        const int idx = tid + c * NT;
-        const int r = idx / CPR, ch = idx % CPR;
-        kreg[c] = *reinterpret_cast<const uint4 *>(kbase + (int64_t)(key0 + r) * p.k.st + ch * 8);
-        vreg[c] = *reinterpret_cast<const uint4 *>(vbase + (int64_t)(key0 + r) * p.v.st + ch * 8);
-      }
-    } else {
-#pragma unroll
-      for (int c = 0; c < CHUNKS; ++c) {
-        const int idx = tid + c * NT;
-        const int r = idx / CPR, ch = idx % CPR;
-        kreg[c] = vreg[c] = make_uint4(0, 0, 0, 0);
-        if (col >= 0 && key0 + r < sq.k_len) {
-          kreg[c] = *reinterpret_cast<const uint4 *>(kbase + (int64_t)(key0 + r) * p.k.st + ch * 8);
-          vreg[c] = *reinterpret_cast<const uint4 *>(vbase + (int64_t)(key0 + r) * p.v.st + ch * 8);
-        }
-      }
-    }
-  };
-  auto commit = [&](int stage) {
-    char *ks = smem + stage * S::kStage, *vs = ks + S::kKBytes;
-#pragma unroll
-    for (int c = 0; c < CHUNKS; ++c) {
-      const int idx = tid + c * NT;
-      const int r = idx / CPR, ch = idx % CPR;
-      *reinterpret_cast<uint4 *>(ks + r * S::kKStride + ch * 16) = kreg[c];
-      *reinterpret_cast<uint4 *>(vs + r * S::kVStride + ch * 16) = vreg[c];
-    }
+    const int valid = col < 0 ? 0 : sq.k_len - key0;
+    char *ks = smem + stage * S::kStage;
+    kload.issue(reinterpret_cast<const char *>(kbase + (int64_t)key0 * p.k.st), 0, valid, ks);
+    vload.issue(reinterpret_cast<const char *>(vbase + (int64_t)key0 * p.v.st), 0, valid, ks + TL::kBytes);
   };
 
   floatx16 oacc[DT];
@@ -128,21 +99,23 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
     for (int r = 0; r < 16; ++r) oacc[dt][r] = 0.f;
   float m_run = -INFINITY, l_run = 0.f;  // running max (log2 domain) and sum of row `pos`
 
-  // LDS offsets of this lane's operand reads
-  const int k_read = m * S::kKStride + g * 16;  // + nt*32 rows + ks*32 bytes
-  const int i16 = lane & 15, dgrp = (lane >> 4) & 1;
-  const int v_read = (4 * g + (i16 >> 2)) * S::kVStride + (16 * dgrp + 4 * (i16 & 3)) * 2;
+  // loop-invariant LDS offsets of this lane's operand reads (row m of a 32-key tile, swizzled
+  // chunk 2ks+g; transpose-read pairs of d-tile dt); tile / k-step row offsets are immediates
+  int rd[KS], tr[DT][2];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) rd[ks] = TL::off(m, 2 * ks + g);
+  transposed_offsets<D>(lane, tr);
 
-  if (e0 < e1) prefetch(e0);
+  if (e0 < e1) issue(e0, 0);
   for (int e = e0; e < e1; ++e) {
     const int stage = (e - e0) & 1;
     const int col = cols[e];
-    commit(stage);
-    __syncthreads();
-    if (e + 1 < e1) prefetch(e + 1);
+    wait_tile_loads();
+    __syncthreads();  // tile e is visible; every wave is done with the other stage
+    if (e + 1 < e1) issue(e + 1, stage ^ 1);
     const int key0 = col * 64;
     if (col < 0 || key0 >= sq.k_len || (p.causal && key0 > row0 + 31)) continue;  // nothing visible (wave-uniform)
-    const char *ks_ = smem + stage * S::kStage, *vs_ = ks_ + S::kKBytes;
+    const char *ks_ = smem + stage * S::kStage, *vs_ = ks_ + TL::kBytes;
 
     // S^T = K Q^T : two 32-key tiles.  Operand reads run one tile ahead of the
     // multiplies so that LDS latency is hidden behind the MFMA pipe.
@@ -158,16 +131,15 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
     {
       vec8 ka[2][KS];
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) ka[0][ks] = lds_read8<vec8>(ks_ + k_read + ks * 32);
+      for (int ks = 0; ks < KS; ++ks) ka[0][ks] = lds_read8<vec8>(ks_ + rd[ks]);
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) ka[1][ks] = lds_read8<vec8>(ks_ + k_read + 32 * S::kKStride + ks * 32);
+      for (int ks = 0; ks < KS; ++ks) ka[1][ks] = lds_read8<vec8>(ks_ + 32 * TL::kRowBytes + rd[ks]);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) sacc[0] = M::mma(ka[0][ks], qf[ks], sacc[0]);
       // first V^T operands do not depend on the softmax: fetch them behind the multiplies
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
-        va[0][dt] = lds_read_tr8<vec8>(vs_ + v_read + dt * 64, vs_ + v_read + 8 * S::kVStride + dt * 64);
+      for (int dt = 0; dt < DT; ++dt) va[0][dt] = lds_read_tr8<vec8>(vs_ + tr[dt][0], vs_ + tr[dt][1]);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) sacc[1] = M::mma(ka[1][ks], qf[ks], sacc[1]);
@@ -226,10 +198,9 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
       for (int i = 0; i < 8; ++i) pf[i] = sacc[nt][t * 8 + i];
       const vec8 pb = M::pack(pf);
       if (step < 3) {
-        const char *vrow = vs_ + v_read + ((step + 1) * 16) * S::kVStride;
+        const char *vrow = vs_ + ((step + 1) * 16) * TL::kRowBytes;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-          va[(step + 1) & 1][dt] = lds_read_tr8<vec8>(vrow + dt * 64, vrow + 8 * S::kVStride + dt * 64);
+        for (int dt = 0; dt < DT; ++dt) va[(step + 1) & 1][dt] = lds_read_tr8<vec8>(vrow + tr[dt][0], vrow + tr[dt][1]);
       }
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) oacc[dt] = M::mma(va[step & 1][dt], pb, oacc[dt]);
@@ -258,6 +229,18 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
     p.lse.ptr[sq.b * p.lse.sb + h * p.lse.sh + (int64_t)(sq.q_start + qi) * p.lse.st] = lse;
   }
 }
+
+// Explicit instantiations: with only the implicit ones the fp16 host stubs of
+// this kernel are not emitted by this compiler version.
+#define DK_INSTANTIATE_FWD(T, D)                                                  \
+  template __global__ void mfma_fwd_kernel<T, D, 1>(const FwdParams, int);       \
+  template __global__ void mfma_fwd_kernel<T, D, 2>(const FwdParams, int);       \
+  template __global__ void mfma_fwd_kernel<T, D, 4>(const FwdParams, int);
+DK_INSTANTIATE_FWD(bf16_t, 128)
+DK_INSTANTIATE_FWD(bf16_t, 64)
+DK_INSTANTIATE_FWD(f16_t, 128)
+DK_INSTANTIATE_FWD(f16_t, 64)
+#undef DK_INSTANTIATE_FWD
 
 // Largest G in {4, 2, 1} such that G consecutive q heads share the kv head and
 // the look-up-table row.

@@ -202,6 +202,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 // ---------------------------------------------------------------------------
 // dK / dV pass
 // ---------------------------------------------------------------------------
+// The dK/dV pass is bound by the latency of its Q / dO tile loads unless several tiles are in
+// flight: 4 LDS stages (133 KB at head_dim 128), one workgroup per CU.
+constexpr int kDkdvStages = 4;
+
 template <typename T, int D>
 __global__ __launch_bounds__(256) void mfma_dkdv_kernel(const BwdParams p) {
   using M = Mma<T>;
@@ -209,7 +213,9 @@ __global__ __launch_bounds__(256) void mfma_dkdv_kernel(const BwdParams p) {
   using TL = Tile<D>;
   constexpr int NT = 256;
   constexpr int KS = D / 16, DT = D / 32;
-  constexpr int STAGE = 2 * TL::kBytes + 512;  // Q tile, dO tile, lse2[64], delta[64]
+  constexpr int STAGE = 2 * TL::kBytes + 512;  // Q tile, dO tile, lse[64], delta[64]
+  constexpr int STAGES = kDkdvStages;          // tiles are requested STAGES - 1 entries ahead
+  constexpr int LPT = 2 * TileLoader<D, NT>::kChunks + 1;  // load instructions per wave per stage
   extern __shared__ __align__(16) char smem[];
 
   const SeqInfo sq = load_seq(p.seqs, blockIdx.z, p.causal);
@@ -217,7 +223,8 @@ __global__ __launch_bounds__(256) void mfma_dkdv_kernel(const BwdParams p) {
   if (cb * 64 >= sq.k_len) return;
   const int kvh = blockIdx.x;
   const int ratio = p.Hq / p.Hkv;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int nh = wave & 1, mh = wave >> 1;
   const int n = lane & 31, g = lane >> 5;
   const int key = cb * 64 + nh * 32 + n;
@@ -244,7 +251,6 @@ __global__ __launch_bounds__(256) void mfma_dkdv_kernel(const BwdParams p) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) dk[dt][r] = dv[dt][r] = 0.f;
 
-  float lreg = 0.f;  // threads 0..63: lse2 of row tid, threads 64..127: delta of row tid-64
   TileLoader<D, NT> qload, doload;
   qload.init(tid, p.q.st);
   doload.init(tid, p.dout.st);
@@ -267,39 +273,50 @@ __global__ __launch_bounds__(256) void mfma_dkdv_kernel(const BwdParams p) {
     const float *lsebase = p.lse.ptr + sq.b * p.lse.sb + h * p.lse.sh;
     const float *deltabase = p.delta + ((int64_t)sq.b * p.Hq + h) * p.seqs.max_q_len;
 
-    // asynchronous copy of q block rows[e] (Q and dO tiles) into `stage`; lse / delta of
-    // its 64 rows are fetched into one register per thread and stored by `commit`
-    auto issue = [&](int e, int stage) {
+    // asynchronous copy of q block rows[e] into `stage`: Q and dO tiles, and the 64 lse / 64
+    // delta values of its rows (threads 0..63 / 64..127; the upper half of the workgroup repeats
+    // the lse load so that every wave issues the same number of load instructions).  Returns
+    // false when rows had to be zero-filled, i.e. when the per-wave load count is not LPT.
+    auto issue = [&](int e, int stage) -> bool {
+      typedef __attribute__((address_space(3))) void *lds_ptr;
       const int rbq = rows[e];
       const int qi0 = rbq * 64 - sq.past;  // query index of the tile's first row
       // rows before the first query (qi < 0, when k is longer than q) and beyond the last are zero-filled
       const int lo = rbq < 0 ? 64 : -qi0, hi = sq.q_len - qi0;
       char *qs = smem + stage * STAGE;
-      qload.issue(reinterpret_cast<const char *>(qbase + (int64_t)qi0 * p.q.st), lo, hi, qs);
+      const bool full = qload.issue(reinterpret_cast<const char *>(qbase + (int64_t)qi0 * p.q.st), lo, hi, qs);
       doload.issue(reinterpret_cast<const char *>(dobase + (int64_t)qi0 * p.dout.st), lo, hi, qs + TL::kBytes);
-      if (tid < 128) {
-        const int qi = qi0 + (tid & 63);
-        const bool ok = rbq >= 0 && qi >= 0 && qi < sq.q_len;
-        if (tid < 64) {
-          const float l = ok ? lsebase[(int64_t)qi * p.lse.st] : -INFINITY;
-          lreg = l == -INFINITY ? INFINITY : l * kLog2e;
-        } else {
-          lreg = ok ? deltabase[qi] : 0.f;
-        }
+      // wave w (of 4) fills floats [64 * (w & 1), +64) of the row-vector area: lse then delta
+      const int row = lane, qi = qi0 + row;
+      const bool is_delta = (wave & 1) != 0;
+      char *dst = qs + 2 * TL::kBytes + (is_delta ? 256 : 0);
+      const float *src = is_delta ? deltabase + qi : lsebase + (int64_t)qi * p.lse.st;
+      if (full) {
+        __builtin_amdgcn_global_load_lds(src, (lds_ptr)dst, 4, 0, 0);
+      } else if (wave < 2) {
+        // rows outside the sequence: lse = +inf makes their probabilities 0
+        float x = is_delta ? 0.f : INFINITY;
+        if (row >= lo && row < hi) x = *src;
+        reinterpret_cast<float *>(dst)[row] = x;
       }
-    };
-    auto commit = [&](int stage) {
-      if (tid < 128) reinterpret_cast<float *>(smem + stage * STAGE + 2 * TL::kBytes)[tid] = lreg;
+      return full;
     };
 
-    if (e0 < e1) issue(e0, 0);
-    for (int e = e0; e < e1; ++e) {
-      const int stage = (e - e0) & 1;
+    int issued = e0, issue_stage = 0, stage = 0;
+    bool exact = true;  // every wave has issued exactly LPT load instructions per outstanding tile
+    for (int i = 0; i < STAGES - 1 && issued < e1; ++i, ++issued) {
+      exact = issue(issued, issue_stage) && exact;
+      issue_stage = issue_stage + 1 == STAGES ? 0 : issue_stage + 1;
+    }
+    for (int e = e0; e < e1; ++e, stage = stage + 1 == STAGES ? 0 : stage + 1) {
       const int rbq = rows[e];
-      wait_tile_loads();
-      commit(stage);
-      __syncthreads();  // tile e is visible; every wave is done with the other stage
-      if (e + 1 < e1) issue(e + 1, stage ^ 1);
+      wait_tiles_ahead<LPT>(exact ? issued - e - 1 : 0);
+      __syncthreads();  // tile e is visible; every wave is done with the stage of tile e - 1
+      if (issued < e1) {
+        exact = issue(issued, issue_stage) && exact;
+        issue_stage = issue_stage + 1 == STAGES ? 0 : issue_stage + 1;
+        ++issued;
+      }
       const int pos0 = rbq * 64 + mh * 32;  // first q position of this wave's half
       if (rbq < 0 || pos0 >= sq.past + sq.q_len || pos0 + 32 <= sq.past) continue;
       if (p.causal && pos0 + 31 < cb * 64 + nh * 32) continue;  // every row above every key of this wave
@@ -331,7 +348,11 @@ __global__ __launch_bounds__(256) void mfma_dkdv_kernel(const BwdParams p) {
         // registers 4*r4 .. +3 are q rows mh*32 + 8*r4 + 4g + {0..3}
         const float4 l4 = *reinterpret_cast<const float4 *>(lse_s + mh * 32 + r4 * 8 + g * 4);
         const float4 d4 = *reinterpret_cast<const float4 *>(delta_s + mh * 32 + r4 * 8 + g * 4);
-        const float lv[4] = {l4.x, l4.y, l4.z, l4.w}, dl[4] = {d4.x, d4.y, d4.z, d4.w};
+        // natural-log lse -> log2 domain; rows that saw no key (-inf) must give p = 0
+        const float lr[4] = {l4.x, l4.y, l4.z, l4.w}, dl[4] = {d4.x, d4.y, d4.z, d4.w};
+        float lv[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) lv[i] = lr[i] == -INFINITY ? INFINITY : lr[i] * kLog2e;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int r = r4 * 4 + i;
@@ -422,7 +443,7 @@ template <typename T, int D>
 static int launch_bwd_td(const BwdParams &p, hipStream_t stream) {
   const SeqView &s = p.seqs;
   constexpr int smem_dq = 2 * 2 * Tile<D>::kBytes;
-  constexpr int smem_dkdv_stage = 2 * (2 * Tile<D>::kBytes + 512);
+  constexpr int smem_dkdv_stage = kDkdvStages * (2 * Tile<D>::kBytes + 512);
   constexpr int smem_red = 2 * 2 * (D / 32) * 16 * 64 * 4;
   constexpr int smem_dkdv = smem_dkdv_stage > smem_red ? smem_dkdv_stage : smem_red;
   static bool attr_set = false;

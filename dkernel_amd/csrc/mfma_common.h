@@ -147,14 +147,16 @@ struct TileLoader {
       goff[c] = (uint32_t)(r * row_stride_elems) * 2u + (uint32_t)((pos ^ Tile<D>::swz(r)) << 4);
     }
   }
-  // rows [lo, hi) of the block are copied, the others zero-filled
-  __device__ __forceinline__ void issue(const char *gblk, int lo, int hi, char *tile) const {
+  // rows [lo, hi) of the block are copied, the others zero-filled.  Returns true when the
+  // whole tile was copied, i.e. when every wave issued exactly kChunks load instructions.
+  __device__ __forceinline__ bool issue(const char *gblk, int lo, int hi, char *tile) const {
     typedef __attribute__((address_space(3))) void *lds_ptr;
     if (lo <= 0 && hi >= 64) {
 #pragma unroll
       for (int c = 0; c < kChunks; ++c)
         __builtin_amdgcn_global_load_lds(gblk + goff[c], (lds_ptr)(tile + (row0 + c * (NT / kCPR)) * Tile<D>::kRowBytes),
                                          16, 0, 0);
+      return true;
     } else {
 #pragma unroll
       for (int c = 0; c < kChunks; ++c) {
@@ -165,12 +167,30 @@ struct TileLoader {
         else
           *reinterpret_cast<uint4 *>(wbase + lane_byte) = make_uint4(0, 0, 0, 0);
       }
+      return false;
     }
   }
 };
 
 // All asynchronous tile loads (and any other vector memory loads) of this wave have landed.
 __device__ __forceinline__ void wait_tile_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+// Multi-stage pipelines: wait until at most `ahead` later tiles (LPT vector
+// memory instructions per wave each) are still in flight, i.e. until the
+// oldest tile has landed.  Vector memory loads return in order.  `ahead` is
+// wave-uniform and at most 3.
+template <int LPT>
+__device__ __forceinline__ void wait_tiles_ahead(int ahead) {
+  static_assert(3 * LPT <= 63, "vmcnt is a 6-bit counter");
+  if (ahead <= 0)
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  else if (ahead == 1)
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LPT) : "memory");
+  else if (ahead == 2)
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * LPT) : "memory");
+  else
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * LPT) : "memory");
+}
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 

@@ -278,7 +278,6 @@ __global__ __launch_bounds__(256) void mfma_dkdv_kernel(const BwdParams p) {
     // the lse load so that every wave issues the same number of load instructions).  Returns
     // false when rows had to be zero-filled, i.e. when the per-wave load count is not LPT.
     auto issue = [&](int e, int stage) -> bool {
-      typedef __attribute__((address_space(3))) void *lds_ptr;
       const int rbq = rows[e];
       const int qi0 = rbq * 64 - sq.past;  // query index of the tile's first row
       // rows before the first query (qi < 0, when k is longer than q) and beyond the last are zero-filled
@@ -292,7 +291,10 @@ __global__ __launch_bounds__(256) void mfma_dkdv_kernel(const BwdParams p) {
       char *dst = qs + 2 * TL::kBytes + (is_delta ? 256 : 0);
       const float *src = is_delta ? deltabase + qi : lsebase + (int64_t)qi * p.lse.st;
       if (full) {
-        __builtin_amdgcn_global_load_lds(src, (lds_ptr)dst, 4, 0, 0);
+        // wave-uniform base (row qi0) + this lane's row
+        const float *src0 = is_delta ? deltabase + qi0 : lsebase + (int64_t)qi0 * p.lse.st;
+        const uint32_t voff = (uint32_t)(row * (is_delta ? 1 : (int)p.lse.st)) * 4u;
+        lds_dma4(reinterpret_cast<const char *>(src0), voff, lds_address(dst));
       } else if (wave < 2) {
         // rows outside the sequence: lse = +inf makes their probabilities 0
         float x = is_delta ? 0.f : INFINITY;

@@ -33,6 +33,7 @@ struct Mma;  // 16-bit element type -> operand vector, MFMA, conversion
 template <>
 struct Mma<bf16_t> {
   using vec8 = bf16x8;
+  using elem = __bf16;
   static __device__ __forceinline__ floatx16 mma(vec8 a, vec8 b, floatx16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
@@ -47,6 +48,7 @@ struct Mma<bf16_t> {
 template <>
 struct Mma<f16_t> {
   using vec8 = f16x8;
+  using elem = _Float16;
   static __device__ __forceinline__ floatx16 mma(vec8 a, vec8 b, floatx16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
   }
@@ -119,8 +121,44 @@ __device__ __forceinline__ void transposed_offsets(int lane, int (&off)[D / 32][
   }
 }
 
+// LDS DMA (global_load_lds): each active lane i of the wave copies `bytes`
+// (16 or 4) from gbase + voff to LDS address lds_base + i * bytes; gbase and
+// lds_base are wave-uniform.  Issued as inline assembly on purpose: for the
+// builtin the compiler places "s_waitcnt vmcnt(0)" in front of every later
+// LDS read (it cannot tell which LDS bytes a copy in flight will write), which
+// serialises a prefetch with the reads of the tile before it.  Here the caller
+// owns the ordering: wait_tile_loads / wait_tiles_ahead, then a barrier,
+// before anything reads what was copied.  Vector memory operations complete in
+// order, so the compiler's own vmcnt bookkeeping for ordinary loads stays
+// conservative (it can only wait for more than it asked for).
+__device__ __forceinline__ uint32_t lds_address(const void *p) {
+  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char *)p;
+}
+// M0 (the LDS base of the copy) is written without telling the compiler: it
+// rejects M0 as a clobber, and nothing else in these kernels uses M0 (on gfx950
+// only LDS DMA, lane-indexed moves and messages read it).
+__device__ __forceinline__ uint64_t uniform_address(const void *p) {
+  // the builtin returns a signed int: narrow to 32 unsigned bits before widening
+  const uint64_t a = (uint64_t)p;
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)a);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+  return ((uint64_t)hi << 32) | (uint64_t)lo;
+}
+__device__ __forceinline__ void lds_dma16(const char *gbase, uint32_t voff, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               :
+               : "v"(voff), "s"(uniform_address(gbase)), "s"(__builtin_amdgcn_readfirstlane(lds_base))
+               : "memory");
+}
+__device__ __forceinline__ void lds_dma4(const char *gbase, uint32_t voff, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
+               :
+               : "v"(voff), "s"(uniform_address(gbase)), "s"(__builtin_amdgcn_readfirstlane(lds_base))
+               : "memory");
+}
+
 // Asynchronous global -> LDS copy of one tile by NT threads, straight into LDS
-// (no staging registers, no ds_write): a wave instruction moves 64 x 16 bytes
+// (LDS DMA: no staging registers, no ds_write): a wave instruction moves 64 x 16 bytes
 // to 1 KB of consecutive LDS; the swizzle is realised by choosing which global
 // chunk each lane fetches (lane position p of row r fetches chunk p ^ swz(r)).
 // TileLoader::init computes the per-thread global byte offsets once.  Rows
@@ -149,13 +187,12 @@ struct TileLoader {
   }
   // rows [lo, hi) of the block are copied, the others zero-filled.  Returns true when the
   // whole tile was copied, i.e. when every wave issued exactly kChunks load instructions.
+  // gblk (first byte of the 64-row block) is wave-uniform.
   __device__ __forceinline__ bool issue(const char *gblk, int lo, int hi, char *tile) const {
-    typedef __attribute__((address_space(3))) void *lds_ptr;
+    const uint32_t base = lds_address(tile) + row0 * Tile<D>::kRowBytes;
     if (lo <= 0 && hi >= 64) {
 #pragma unroll
-      for (int c = 0; c < kChunks; ++c)
-        __builtin_amdgcn_global_load_lds(gblk + goff[c], (lds_ptr)(tile + (row0 + c * (NT / kCPR)) * Tile<D>::kRowBytes),
-                                         16, 0, 0);
+      for (int c = 0; c < kChunks; ++c) lds_dma16(gblk, goff[c], base + c * (NT / kCPR) * Tile<D>::kRowBytes);
       return true;
     } else {
 #pragma unroll
@@ -163,7 +200,7 @@ struct TileLoader {
         char *wbase = tile + (row0 + c * (NT / kCPR)) * Tile<D>::kRowBytes;
         const int r = row0 + c * (NT / kCPR) + lane_row;
         if (r >= lo && r < hi)
-          __builtin_amdgcn_global_load_lds(gblk + goff[c], (lds_ptr)wbase, 16, 0, 0);
+          lds_dma16(gblk, goff[c], base + c * (NT / kCPR) * Tile<D>::kRowBytes);
         else
           *reinterpret_cast<uint4 *>(wbase + lane_byte) = make_uint4(0, 0, 0, 0);
       }
@@ -197,5 +234,17 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 // Exchange with the lane 32 away (the other half-wave that holds the rest of
 // an accumulator row).
 __device__ __forceinline__ float xor32(float x) { return __shfl_xor(x, 32); }
+
+// The same exchange as one VALU instruction (no LDS round trip): v_permlane32_swap
+// trades the upper half of its first operand for the lower half of its second,
+// so (x, x) yields {lo, lo} and {hi, hi}; a lane's partner value is the one that
+// differs from its own.  Returned for use in a symmetric reduction: the result is
+// max/sum-equivalent to xor32 when combined with the lane's own value.
+__device__ __forceinline__ float xor32_swap(float x) {
+  const unsigned u = __builtin_bit_cast(unsigned, x);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  // lanes 0..31 hold their own value in r[0] and the partner's in r[1]; lanes 32..63 the reverse
+  return __builtin_bit_cast(float, (threadIdx.x & 32) ? r[0] : r[1]);
+}
 
 }  // namespace dk

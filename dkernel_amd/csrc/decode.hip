@@ -59,7 +59,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
   const int unit = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
   const SeqInfo sq = load_seq(p.seqs, b, p.causal);
   if (sq.q_len <= 0 || sq.k_len <= 0) return;
-  const int ratio = p.Hq / p.Hkv;
+  const int ratio = __builtin_amdgcn_readfirstlane(p.Hq / p.Hkv);  // integer division runs on the VALU
   const int lane = threadIdx.x;
   const int m = lane & 31, g = lane >> 5;  // m = q head inside the group (MFMA column)
   const int pos = sq.past;                 // absolute position of the single query token

@@ -78,11 +78,11 @@ struct BwdParams {
   int32_t vec_ok;
 };
 
-// Which LUT head serves q head h.
+// Which LUT head serves q head h (h is the same for every lane of a wave).
 __device__ __forceinline__ int lut_head(const LutView &l, int h, int Hq, int Hkv) {
   if (l.num_heads == 1) return 0;
   if (l.num_heads == Hq) return h;
-  return h / (Hq / Hkv);
+  return __builtin_amdgcn_readfirstlane(h / (Hq / Hkv));  // integer division runs on the VALU
 }
 
 struct SeqInfo {
@@ -109,6 +109,13 @@ __device__ __forceinline__ SeqInfo load_seq(const SeqView &s, int b, int causal)
   if (r.k_len < 0) r.k_len = 0;
   r.past = causal ? r.k_len - r.q_len : 0;
   if (r.past < 0) r.past = 0;
+  // b is the same for every lane of a wave, so the fields are too; saying so keeps the
+  // addresses derived from them in scalar registers
+  r.q_start = __builtin_amdgcn_readfirstlane(r.q_start);
+  r.q_len = __builtin_amdgcn_readfirstlane(r.q_len);
+  r.k_start = __builtin_amdgcn_readfirstlane(r.k_start);
+  r.k_len = __builtin_amdgcn_readfirstlane(r.k_len);
+  r.past = __builtin_amdgcn_readfirstlane(r.past);
   return r;
 }
 

@@ -45,7 +45,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int rh = wave & 1, kh = wave >> 1;  // q-row half, key half
   const int h = blockIdx.x;
-  const int kvh = h / (p.Hq / p.Hkv);
+  const int kvh = __builtin_amdgcn_readfirstlane(h / (p.Hq / p.Hkv));  // integer division runs on the VALU
   const int m = lane & 31, g = lane >> 5;
   const int row0 = rb * 64 + rh * 32;
   const int pos = row0 + m;
@@ -202,54 +202,77 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 // ---------------------------------------------------------------------------
 // dK / dV pass
 // ---------------------------------------------------------------------------
-// The dK/dV pass is bound by the latency of its Q / dO tile loads unless several tiles are in
-// flight: 4 LDS stages (133 KB at head_dim 128), one workgroup per CU.
-constexpr int kDkdvStages = 4;
+// One workgroup = one 64-key column block of one kv head, 8 waves.  The four
+// 32 x 32 (q rows x keys) quadrants of a block are each worked on by a pair of
+// waves that sit on the same SIMD:
+//   the S wave:   S = Q K^T, P = exp(S - lse), dV^T += dO^T P     (K fragments and dV in registers)
+//   the dP wave:  dP = dO V^T, dS = P (dP - delta), dK^T += Q^T dS (V fragments and dK in registers)
+// so that each wave holds half of the accumulators and fits in the 256
+// registers of two waves per SIMD.  P goes from the S wave to the dP wave
+// through LDS in fp32, exactly as computed.  The dP wave finishes a block one
+// iteration late (after the next block's barrier has published P), so one
+// barrier per block is enough: Q tiles and the lse / delta vectors live one
+// iteration longer than dO tiles (rings of 4 and 3 stages), and tile loads run
+// two blocks ahead.
+template <bool V>
+struct BoolConst {
+  static constexpr bool value = V;
+};
+
+template <int D>
+struct DkdvSmem {
+  using TL = Tile<D>;
+  static constexpr int kQStages = 4, kDoStages = 3, kAhead = 2;
+  static constexpr int kQ = 0;                                // Q ring
+  static constexpr int kDo = kQ + kQStages * TL::kBytes;      // dO ring
+  static constexpr int kVec = kDo + kDoStages * TL::kBytes;   // per Q stage: lse[64], delta[64]
+  static constexpr int kX = kVec + kQStages * 512;            // P exchange: [pair 4][buffer 2][16][64] floats
+  static constexpr int kLoop = kX + 4 * 2 * 4096;
+  static constexpr int kRed = 2 * 2 * (D / 32) * 16 * 64 * 4;  // epilogue: [role][nh][DT*16][64] floats
+  static constexpr int kBytes = kLoop > kRed ? kLoop : kRed;
+};
 
 template <typename T, int D>
-__global__ __launch_bounds__(256) void mfma_dkdv_kernel(const BwdParams p) {
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void mfma_dkdv_kernel(const BwdParams p) {
   using M = Mma<T>;
   using vec8 = typename M::vec8;
   using TL = Tile<D>;
-  constexpr int NT = 256;
+  using S = DkdvSmem<D>;
+  constexpr int NT = 512;
   constexpr int KS = D / 16, DT = D / 32;
-  constexpr int STAGE = 2 * TL::kBytes + 512;  // Q tile, dO tile, lse[64], delta[64]
-  constexpr int STAGES = kDkdvStages;          // tiles are requested STAGES - 1 entries ahead
-  constexpr int LPT = 2 * TileLoader<D, NT>::kChunks + 1;  // load instructions per wave per stage
+  constexpr int LPT = 2 * TileLoader<D, NT>::kChunks + 1;  // load instructions per wave per block
   extern __shared__ __align__(16) char smem[];
 
   const SeqInfo sq = load_seq(p.seqs, blockIdx.z, p.causal);
   const int cb = blockIdx.y;
   if (cb * 64 >= sq.k_len) return;
   const int kvh = blockIdx.x;
-  const int ratio = p.Hq / p.Hkv;
+  const int ratio = __builtin_amdgcn_readfirstlane(p.Hq / p.Hkv);  // integer division runs on the VALU
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int nh = wave & 1, mh = wave >> 1;
+  const int pair = wave & 3, nh = wave & 1, mh = (wave >> 1) & 1;
+  const bool dp_wave = wave >= 4;
   const int n = lane & 31, g = lane >> 5;
   const int key = cb * 64 + nh * 32 + n;
   const bool key_ok = key < sq.k_len;
 
-  vec8 kf[KS], vf[KS];
+  // K fragments (S wave) or V fragments (dP wave): B operand of the first product
+  vec8 kvf[KS];
   {
-    const T *kp = (const T *)p.k.ptr + sq.b * p.k.sb + kvh * p.k.sh + (int64_t)key * p.k.st;
-    const T *vp = (const T *)p.v.ptr + sq.b * p.v.sb + kvh * p.v.sh + (int64_t)key * p.v.st;
+    const T *src = dp_wave ? (const T *)p.v.ptr + sq.b * p.v.sb + kvh * p.v.sh + (int64_t)key * p.v.st
+                           : (const T *)p.k.ptr + sq.b * p.k.sb + kvh * p.k.sh + (int64_t)key * p.k.st;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      uint4 a = make_uint4(0, 0, 0, 0), b = a;
-      if (key_ok) {
-        a = *reinterpret_cast<const uint4 *>(kp + ks * 16 + g * 8);
-        b = *reinterpret_cast<const uint4 *>(vp + ks * 16 + g * 8);
-      }
-      kf[ks] = as_vec8<vec8>(a);
-      vf[ks] = as_vec8<vec8>(b);
+      uint4 a = make_uint4(0, 0, 0, 0);
+      if (key_ok) a = *reinterpret_cast<const uint4 *>(src + ks * 16 + g * 8);
+      kvf[ks] = as_vec8<vec8>(a);
     }
   }
-  floatx16 dk[DT], dv[DT];
+  floatx16 acc[DT];  // dV^T (S wave) or dK^T (dP wave): d x keys
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) dk[dt][r] = dv[dt][r] = 0.f;
+    for (int r = 0; r < 16; ++r) acc[dt][r] = 0.f;
 
   TileLoader<D, NT> qload, doload;
   qload.init(tid, p.q.st);
@@ -258,6 +281,7 @@ __global__ __launch_bounds__(256) void mfma_dkdv_kernel(const BwdParams p) {
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) rd[ks] = TL::off(mh * 32 + n, 2 * ks + g);
   transposed_offsets<D>(lane, tr);
+  float *xbuf = reinterpret_cast<float *>(smem + S::kX) + pair * 2 * 1024;  // this pair's two P buffers
 
   for (int gq = 0; gq < ratio; ++gq) {
     const int h = kvh * ratio + gq;
@@ -267,29 +291,29 @@ __global__ __launch_bounds__(256) void mfma_dkdv_kernel(const BwdParams p) {
       e0 = p.csc.ptr[lh * p.csc.ptr_sh + cb];
       e1 = p.csc.ptr[lh * p.csc.ptr_sh + cb + 1];
     }
-    const int32_t *rows = p.csc.idx + lh * p.csc.idx_sh;
+    const int nblk = __builtin_amdgcn_readfirstlane(e1 - e0);
+    const int32_t *rows = p.csc.idx + lh * p.csc.idx_sh + e0;
     const T *qbase = (const T *)p.q.ptr + sq.b * p.q.sb + h * p.q.sh;
     const T *dobase = (const T *)p.dout.ptr + sq.b * p.dout.sb + h * p.dout.sh;
     const float *lsebase = p.lse.ptr + sq.b * p.lse.sb + h * p.lse.sh;
     const float *deltabase = p.delta + ((int64_t)sq.b * p.Hq + h) * p.seqs.max_q_len;
 
-    // asynchronous copy of q block rows[e] into `stage`: Q and dO tiles, and the 64 lse / 64
-    // delta values of its rows (threads 0..63 / 64..127; the upper half of the workgroup repeats
-    // the lse load so that every wave issues the same number of load instructions).  Returns
-    // false when rows had to be zero-filled, i.e. when the per-wave load count is not LPT.
-    auto issue = [&](int e, int stage) -> bool {
-      const int rbq = rows[e];
+    // asynchronous copy of q block rows[t]: Q and dO tiles and the 64 lse / 64 delta values of
+    // its rows (even waves copy lse, odd waves delta; they all write the same values, so that
+    // every wave issues the same number of load instructions).  Returns false when rows had
+    // to be zero-filled, i.e. when the per-wave load count is not LPT.
+    auto issue = [&](int t, int qstage, int dostage) -> bool {
+      const int rbq = scalar_load(rows + t);
       const int qi0 = rbq * 64 - sq.past;  // query index of the tile's first row
       // rows before the first query (qi < 0, when k is longer than q) and beyond the last are zero-filled
       const int lo = rbq < 0 ? 64 : -qi0, hi = sq.q_len - qi0;
-      char *qs = smem + stage * STAGE;
-      const bool full = qload.issue(reinterpret_cast<const char *>(qbase + (int64_t)qi0 * p.q.st), lo, hi, qs);
-      doload.issue(reinterpret_cast<const char *>(dobase + (int64_t)qi0 * p.dout.st), lo, hi, qs + TL::kBytes);
-      // wave w (of 4) fills floats [64 * (w & 1), +64) of the row-vector area: lse then delta
-      const int row = lane, qi = qi0 + row;
+      const bool full = qload.issue(reinterpret_cast<const char *>(qbase + (int64_t)qi0 * p.q.st), lo, hi,
+                                    smem + S::kQ + qstage * TL::kBytes);
+      doload.issue(reinterpret_cast<const char *>(dobase + (int64_t)qi0 * p.dout.st), lo, hi,
+                   smem + S::kDo + dostage * TL::kBytes);
+      const int row = lane;
       const bool is_delta = (wave & 1) != 0;
-      char *dst = qs + 2 * TL::kBytes + (is_delta ? 256 : 0);
-      const float *src = is_delta ? deltabase + qi : lsebase + (int64_t)qi * p.lse.st;
+      char *dst = smem + S::kVec + qstage * 512 + (is_delta ? 256 : 0);
       if (full) {
         // wave-uniform base (row qi0) + this lane's row
         const float *src0 = is_delta ? deltabase + qi0 : lsebase + (int64_t)qi0 * p.lse.st;
@@ -297,130 +321,176 @@ __global__ __launch_bounds__(256) void mfma_dkdv_kernel(const BwdParams p) {
         lds_dma4(reinterpret_cast<const char *>(src0), voff, lds_address(dst));
       } else if (wave < 2) {
         // rows outside the sequence: lse = +inf makes their probabilities 0
+        const int qi = qi0 + row;
         float x = is_delta ? 0.f : INFINITY;
-        if (row >= lo && row < hi) x = *src;
+        if (row >= lo && row < hi) x = is_delta ? deltabase[qi] : lsebase[(int64_t)qi * p.lse.st];
         reinterpret_cast<float *>(dst)[row] = x;
       }
       return full;
     };
 
-    int issued = e0, issue_stage = 0, stage = 0;
-    bool exact = true;  // every wave has issued exactly LPT load instructions per outstanding tile
-    for (int i = 0; i < STAGES - 1 && issued < e1; ++i, ++issued) {
-      exact = issue(issued, issue_stage) && exact;
-      issue_stage = issue_stage + 1 == STAGES ? 0 : issue_stage + 1;
-    }
-    for (int e = e0; e < e1; ++e, stage = stage + 1 == STAGES ? 0 : stage + 1) {
-      const int rbq = rows[e];
-      wait_tiles_ahead<LPT>(exact ? issued - e - 1 : 0);
-      __syncthreads();  // tile e is visible; every wave is done with the stage of tile e - 1
-      if (issued < e1) {
-        exact = issue(issued, issue_stage) && exact;
-        issue_stage = issue_stage + 1 == STAGES ? 0 : issue_stage + 1;
-        ++issued;
-      }
-      const int pos0 = rbq * 64 + mh * 32;  // first q position of this wave's half
-      if (rbq < 0 || pos0 >= sq.past + sq.q_len || pos0 + 32 <= sq.past) continue;
-      if (p.causal && pos0 + 31 < cb * 64 + nh * 32) continue;  // every row above every key of this wave
-      const char *qs_ = smem + stage * STAGE, *dos_ = qs_ + TL::kBytes;
-      const float *lse_s = reinterpret_cast<const float *>(qs_ + 2 * TL::kBytes);
-      const float *delta_s = lse_s + 64;
-
-      // S = Q K^T, dP = dO V^T : rows = 32 q positions, cols = 32 keys
-      floatx16 s, dp;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) s[r] = dp[r] = 0.f;
-      {
-        vec8 qa[KS], da[KS];
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          qa[ks] = lds_read8<vec8>(qs_ + rd[ks]);
-          da[ks] = lds_read8<vec8>(dos_ + rd[ks]);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          s = M::mma(qa[ks], kf[ks], s);
-          dp = M::mma(da[ks], vf[ks], dp);
-        }
-      }
-      const bool need_mask = p.causal && (cb * 64 + nh * 32 + 31 > pos0);
+    // second half of the dP wave's work on block u (whose P the S wave published before the
+    // last barrier): dS = P (dP - delta), dK^T += Q^T dS
+    auto finish_dk = [&](int u, int qstage, const floatx16 &dp) {
+      const char *qs_ = smem + S::kQ + qstage * TL::kBytes;
+      const float *delta_s = reinterpret_cast<const float *>(smem + S::kVec + qstage * 512) + 64;
+      const float *x = xbuf + (u & 1) * 1024;
+      float ds[16];
 #pragma unroll
       for (int r4 = 0; r4 < 4; ++r4) {
-        // registers 4*r4 .. +3 are q rows mh*32 + 8*r4 + 4g + {0..3}
-        const float4 l4 = *reinterpret_cast<const float4 *>(lse_s + mh * 32 + r4 * 8 + g * 4);
+        const float4 p4 = *reinterpret_cast<const float4 *>(x + (r4 * 64 + lane) * 4);
         const float4 d4 = *reinterpret_cast<const float4 *>(delta_s + mh * 32 + r4 * 8 + g * 4);
-        // natural-log lse -> log2 domain; rows that saw no key (-inf) must give p = 0
-        const float lr[4] = {l4.x, l4.y, l4.z, l4.w}, dl[4] = {d4.x, d4.y, d4.z, d4.w};
-        float lv[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) lv[i] = lr[i] == -INFINITY ? INFINITY : lr[i] * kLog2e;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int r = r4 * 4 + i;
-          float pr = fast_exp2(fmaf(s[r], p.scale_log2, -lv[i]));
-          if (need_mask) pr = key > pos0 + r4 * 8 + g * 4 + i ? 0.f : pr;
-          pr = key_ok ? pr : 0.f;
-          s[r] = pr;                       // P
-          dp[r] = pr * (dp[r] - dl[i]);    // dS without sm_scale
-        }
+        ds[r4 * 4 + 0] = p4.x * (dp[r4 * 4 + 0] - d4.x);  // without sm_scale
+        ds[r4 * 4 + 1] = p4.y * (dp[r4 * 4 + 1] - d4.y);
+        ds[r4 * 4 + 2] = p4.z * (dp[r4 * 4 + 2] - d4.z);
+        ds[r4 * 4 + 3] = p4.w * (dp[r4 * 4 + 3] - d4.w);
       }
 #pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        float pf[8], df[8];
+      for (int t2 = 0; t2 < 2; ++t2) {
+        const vec8 dsb = M::pack(ds + t2 * 8);
+        const int rowoff = (mh * 32 + t2 * 16) * TL::kRowBytes;
+        vec8 qt[DT];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          pf[i] = s[t * 8 + i];
-          df[i] = dp[t * 8 + i];
-        }
-        const vec8 pb = M::pack(pf), dsb = M::pack(df);
-        const int rowoff = (mh * 32 + t * 16) * TL::kRowBytes;
-        vec8 dot[DT], qt[DT];
+        for (int dt = 0; dt < DT; ++dt) qt[dt] = lds_read_tr8<vec8>(qs_ + rowoff + tr[dt][0], qs_ + rowoff + tr[dt][1]);
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-          dot[dt] = lds_read_tr8<vec8>(dos_ + rowoff + tr[dt][0], dos_ + rowoff + tr[dt][1]);
-          qt[dt] = lds_read_tr8<vec8>(qs_ + rowoff + tr[dt][0], qs_ + rowoff + tr[dt][1]);
-        }
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-          dv[dt] = M::mma(dot[dt], pb, dv[dt]);
-          dk[dt] = M::mma(qt[dt], dsb, dk[dt]);
-        }
+        for (int dt = 0; dt < DT; ++dt) acc[dt] = M::mma(qt[dt], dsb, acc[dt]);
       }
+    };
+
+    // The loop is instantiated once per role (not branched inside), so that the accumulators
+    // are not merged through a join every iteration.
+    auto run_head = [&](auto role_tag) {
+    constexpr bool kDp = decltype(role_tag)::value;
+    int issued = 0, iq = 0, ido = 0;  // next block to request and its ring positions
+    bool exact = true;                // every wave has issued exactly LPT load instructions per outstanding block
+    for (int i = 0; i < S::kAhead && issued < nblk; ++i, ++issued) {
+      exact = issue(issued, iq, ido) && exact;
+      iq = iq + 1 == S::kQStages ? 0 : iq + 1;
+      ido = ido + 1 == S::kDoStages ? 0 : ido + 1;
     }
-    __syncthreads();  // every wave is done with both stages before the next head reuses them
+    floatx16 dp_prev;
+    int cq = 0, cdo = 0, pq = 0;  // ring positions of block t (Q, dO) and of block t - 1 (Q)
+    for (int t = 0; t < nblk; ++t) {
+      wait_tiles_ahead<LPT>(exact ? issued - t - 1 : 0);
+      __syncthreads();  // block t is visible, so is P of block t - 1; the stages of block t - 2 are free
+      if (issued < nblk) {
+        exact = issue(issued, iq, ido) && exact;
+        iq = iq + 1 == S::kQStages ? 0 : iq + 1;
+        ido = ido + 1 == S::kDoStages ? 0 : ido + 1;
+        ++issued;
+      }
+      const char *qs_ = smem + S::kQ + cq * TL::kBytes, *dos_ = smem + S::kDo + cdo * TL::kBytes;
+      if constexpr (!kDp) {
+        const int rbq = scalar_load(rows + t);
+        const int pos0 = rbq * 64 + mh * 32;  // first q position of this wave's half
+        const float *lse_s = reinterpret_cast<const float *>(smem + S::kVec + cq * 512);
+        // S = Q K^T : rows = 32 q positions, cols = 32 keys
+        floatx16 sc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sc[r] = 0.f;
+        {
+          vec8 qa[KS];
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks) qa[ks] = lds_read8<vec8>(qs_ + rd[ks]);
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks) sc = M::mma(qa[ks], kvf[ks], sc);
+        }
+        // first dO^T operands do not depend on P
+        vec8 dot[DT];
+        {
+          const int rowoff = (mh * 32) * TL::kRowBytes;
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt) dot[dt] = lds_read_tr8<vec8>(dos_ + rowoff + tr[dt][0], dos_ + rowoff + tr[dt][1]);
+        }
+        const bool need_mask = p.causal && (cb * 64 + nh * 32 + 31 > pos0);
+        float *x = xbuf + (t & 1) * 1024;
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) {
+          // registers 4*r4 .. +3 are q rows mh*32 + 8*r4 + 4g + {0..3}
+          const float4 l4 = *reinterpret_cast<const float4 *>(lse_s + mh * 32 + r4 * 8 + g * 4);
+          const float lr[4] = {l4.x, l4.y, l4.z, l4.w};
+          float pr[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            // natural-log lse -> log2 domain; rows that saw no key (-inf) must give p = 0
+            const float lv = lr[i] == -INFINITY ? INFINITY : lr[i] * kLog2e;
+            float v = fast_exp2(fmaf(sc[r4 * 4 + i], p.scale_log2, -lv));
+            if (need_mask) v = key > pos0 + r4 * 8 + g * 4 + i ? 0.f : v;
+            pr[i] = key_ok ? v : 0.f;
+            sc[r4 * 4 + i] = pr[i];
+          }
+          *reinterpret_cast<float4 *>(x + (r4 * 64 + lane) * 4) = make_float4(pr[0], pr[1], pr[2], pr[3]);
+        }
+        // dV^T += dO^T P
+#pragma unroll
+        for (int t2 = 0; t2 < 2; ++t2) {
+          float pf[8];
+#pragma unroll
+          for (int i = 0; i < 8; ++i) pf[i] = sc[t2 * 8 + i];
+          const vec8 pb = M::pack(pf);
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt) {
+            acc[dt] = M::mma(dot[dt], pb, acc[dt]);
+            if (t2 == 0) {
+              const int rowoff = (mh * 32 + 16) * TL::kRowBytes;
+              dot[dt] = lds_read_tr8<vec8>(dos_ + rowoff + tr[dt][0], dos_ + rowoff + tr[dt][1]);
+            }
+          }
+        }
+      } else {
+        // second half of block t - 1 first: it frees dp_prev for this block's dP
+        if (t > 0) finish_dk(t - 1, pq, dp_prev);
+        // dP = dO V^T
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dp_prev[r] = 0.f;
+        {
+          vec8 da[KS];
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks) da[ks] = lds_read8<vec8>(dos_ + rd[ks]);
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks) dp_prev = M::mma(da[ks], kvf[ks], dp_prev);
+        }
+      }
+      pq = cq;
+      cq = cq + 1 == S::kQStages ? 0 : cq + 1;
+      cdo = cdo + 1 == S::kDoStages ? 0 : cdo + 1;
+    }
+    __syncthreads();  // P of the last block is visible
+    if constexpr (kDp) {
+      if (nblk > 0) finish_dk(nblk - 1, pq, dp_prev);
+    }
+    };
+    if (dp_wave)
+      run_head(BoolConst<true>{});
+    else
+      run_head(BoolConst<false>{});
+    __syncthreads();  // every wave is done with every stage before the next head reuses them
   }
 
   // sum the two q-row halves: waves with mh = 1 hand their partials to mh = 0
-  float *red = reinterpret_cast<float *>(smem);
+  float *red = reinterpret_cast<float *>(smem) + ((dp_wave ? 2 : 0) + nh) * DT * 16 * 64;
   if (mh == 1) {
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        red[((nh * 2 + 0) * DT * 16 + dt * 16 + r) * 64 + lane] = dk[dt][r];
-        red[((nh * 2 + 1) * DT * 16 + dt * 16 + r) * 64 + lane] = dv[dt][r];
-      }
+      for (int r = 0; r < 16; ++r) red[(dt * 16 + r) * 64 + lane] = acc[dt][r];
   }
   __syncthreads();
   if (mh == 1 || !key_ok) return;
-  T *dkp = (T *)p.dk.ptr + sq.b * p.dk.sb + kvh * p.dk.sh + (int64_t)key * p.dk.st;
-  T *dvp = (T *)p.dv.ptr + sq.b * p.dv.sb + kvh * p.dv.sh + (int64_t)key * p.dv.st;
+  const float out_scale = dp_wave ? p.sm_scale : 1.f;
+  T *outp = dp_wave ? (T *)p.dk.ptr + sq.b * p.dk.sb + kvh * p.dk.sh + (int64_t)key * p.dk.st
+                    : (T *)p.dv.ptr + sq.b * p.dv.sb + kvh * p.dv.sh + (int64_t)key * p.dv.st;
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
     for (int r4 = 0; r4 < 4; ++r4) {
-      T k4[4], v4[4];
+      T o4[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int r = r4 * 4 + i;
-        const float a = dk[dt][r] + red[((nh * 2 + 0) * DT * 16 + dt * 16 + r) * 64 + lane];
-        const float b = dv[dt][r] + red[((nh * 2 + 1) * DT * 16 + dt * 16 + r) * 64 + lane];
-        k4[i] = from_float<T>(a * p.sm_scale);
-        v4[i] = from_float<T>(b);
+        o4[i] = from_float<T>((acc[dt][r] + red[(dt * 16 + r) * 64 + lane]) * out_scale);
       }
-      *reinterpret_cast<uint2 *>(dkp + dt * 32 + r4 * 8 + g * 4) = *reinterpret_cast<const uint2 *>(k4);
-      *reinterpret_cast<uint2 *>(dvp + dt * 32 + r4 * 8 + g * 4) = *reinterpret_cast<const uint2 *>(v4);
+      *reinterpret_cast<uint2 *>(outp + dt * 32 + r4 * 8 + g * 4) = *reinterpret_cast<const uint2 *>(o4);
     }
 }
 
@@ -445,9 +515,7 @@ template <typename T, int D>
 static int launch_bwd_td(const BwdParams &p, hipStream_t stream) {
   const SeqView &s = p.seqs;
   constexpr int smem_dq = 2 * 2 * Tile<D>::kBytes;
-  constexpr int smem_dkdv_stage = kDkdvStages * (2 * Tile<D>::kBytes + 512);
-  constexpr int smem_red = 2 * 2 * (D / 32) * 16 * 64 * 4;
-  constexpr int smem_dkdv = smem_dkdv_stage > smem_red ? smem_dkdv_stage : smem_red;
+  constexpr int smem_dkdv = DkdvSmem<D>::kBytes;
   static bool attr_set = false;
   if (!attr_set) {
     DK_HIP_CHECK(hipFuncSetAttribute((const void *)mfma_dq_kernel<T, D>,
@@ -460,7 +528,7 @@ static int launch_bwd_td(const BwdParams &p, hipStream_t stream) {
   const int tiles = (past + s.max_q_len - 1) / 64 - past / 64 + 1;
   const int cblocks = cdiv(s.max_k_len, 64);
   DK_REQUIRE(tiles <= 65535 && cblocks <= 65535, "sequence too long for one launch");
-  hipLaunchKernelGGL((mfma_dkdv_kernel<T, D>), dim3(p.Hkv, cblocks, s.batch), dim3(256), smem_dkdv, stream, p);
+  hipLaunchKernelGGL((mfma_dkdv_kernel<T, D>), dim3(p.Hkv, cblocks, s.batch), dim3(512), smem_dkdv, stream, p);
   DK_HIP_CHECK(hipGetLastError());
   hipLaunchKernelGGL((mfma_dq_kernel<T, D>), dim3(p.Hq, tiles, s.batch), dim3(256), smem_dq, stream, p, tiles);
   DK_HIP_CHECK(hipGetLastError());

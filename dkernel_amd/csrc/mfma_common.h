@@ -144,6 +144,15 @@ __device__ __forceinline__ uint64_t uniform_address(const void *p) {
   const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
   return ((uint64_t)hi << 32) | (uint64_t)lo;
 }
+// Read one int32 of a look-up table at a wave-uniform address through the scalar
+// unit.  A vector load here would make the compiler wait for every vector
+// memory operation in flight (vmcnt(0)), tile copies included, before the
+// value can be used.
+__device__ __forceinline__ int scalar_load(const int32_t *p) {
+  int v;
+  asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(v) : "s"(uniform_address(p)) : "memory");
+  return v;
+}
 __device__ __forceinline__ void lds_dma16(const char *gbase, uint32_t voff, uint32_t lds_base) {
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                :

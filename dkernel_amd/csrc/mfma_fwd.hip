@@ -50,7 +50,7 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
   const int rb = sq.past / 64 + tile;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int h = blockIdx.x * G + (wave >> 1);
-  const int kvh = h / (p.Hq / p.Hkv);
+  const int kvh = __builtin_amdgcn_readfirstlane(h / (p.Hq / p.Hkv));  // integer division runs on the VALU
   const int m = lane & 31, g = lane >> 5;
   const int row0 = rb * 64 + (wave & 1) * 32;  // first absolute position of this wave
   const int pos = row0 + m;
@@ -262,7 +262,7 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int h = blockIdx.x * G + (wave >> 1);
-  const int kvh = h / (p.Hq / p.Hkv);
+  const int kvh = __builtin_amdgcn_readfirstlane(h / (p.Hq / p.Hkv));  // integer division runs on the VALU
   const int m = lane & 31, g = lane >> 5;
   const int row0 = rb * 64 + (wave & 1) * 32;
   const int pos = row0 + m;

@@ -17,6 +17,8 @@
 //
 // Tiles are copied HBM -> LDS asynchronously (no staging registers), double
 // buffered, in the swizzled row-major layout of mfma_common.h.
+#include <climits>
+
 #include "common.h"
 #include "device_common.h"
 #include "mfma_common.h"
@@ -402,25 +404,32 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
           for (int dt = 0; dt < DT; ++dt) dot[dt] = lds_read_tr8<vec8>(dos_ + rowoff + tr[dt][0], dos_ + rowoff + tr[dt][1]);
         }
-        const bool need_mask = p.causal && (cb * 64 + nh * 32 + 31 > pos0);
+        // P = exp2(S scale - lse log2e).  Rows outside the sequence arrive with lse = +inf
+        // (P = 0).  A row that saw no key has lse = -inf, but then every one of its entries
+        // here is masked by causality and the select below discards the infinite value, so no
+        // conversion is needed.  Masks are applied only in blocks that need them (the diagonal
+        // block and the last, partial column block): wave-uniform choice between two loops.
+        const bool edge = (p.causal && (cb * 64 + nh * 32 + 31 > pos0)) || cb * 64 + 63 >= sq.k_len;
+        // last visible q-row offset test: key is visible to row pos iff key <= pos
+        const int kcmp = key_ok ? (p.causal ? key - pos0 : INT_MIN) : INT_MAX;  // masked iff kcmp > row offset
         float *x = xbuf + (t & 1) * 1024;
 #pragma unroll
         for (int r4 = 0; r4 < 4; ++r4) {
           // registers 4*r4 .. +3 are q rows mh*32 + 8*r4 + 4g + {0..3}
           const float4 l4 = *reinterpret_cast<const float4 *>(lse_s + mh * 32 + r4 * 8 + g * 4);
           const float lr[4] = {l4.x, l4.y, l4.z, l4.w};
-          float pr[4];
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            // natural-log lse -> log2 domain; rows that saw no key (-inf) must give p = 0
-            const float lv = lr[i] == -INFINITY ? INFINITY : lr[i] * kLog2e;
-            float v = fast_exp2(fmaf(sc[r4 * 4 + i], p.scale_log2, -lv));
-            if (need_mask) v = key > pos0 + r4 * 8 + g * 4 + i ? 0.f : v;
-            pr[i] = key_ok ? v : 0.f;
-            sc[r4 * 4 + i] = pr[i];
-          }
-          *reinterpret_cast<float4 *>(x + (r4 * 64 + lane) * 4) = make_float4(pr[0], pr[1], pr[2], pr[3]);
+          for (int i = 0; i < 4; ++i)
+            sc[r4 * 4 + i] = fast_exp2(fmaf(sc[r4 * 4 + i], p.scale_log2, -lr[i] * kLog2e));
         }
+        if (edge) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) sc[r] = kcmp > (r >> 2) * 8 + g * 4 + (r & 3) ? 0.f : sc[r];
+        }
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4)
+          *reinterpret_cast<float4 *>(x + (r4 * 64 + lane) * 4) =
+              make_float4(sc[r4 * 4], sc[r4 * 4 + 1], sc[r4 * 4 + 2], sc[r4 * 4 + 3]);
         // dV^T += dO^T P
 #pragma unroll
         for (int t2 = 0; t2 < 2; ++t2) {

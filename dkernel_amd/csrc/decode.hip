@@ -42,8 +42,8 @@ template <int D>
 struct DecSmem {  // per wave: one 32-key half block of K and of V, plus q of the group
   static constexpr int kStride = D * 2 + 16;   // bytes per row
   static constexpr int kHalf = 32 * kStride;   // one half-block tile
-  static constexpr int kQBytes = 32 * D * 2;   // q of up to 32 heads, row-major
-  static constexpr int kWave = 2 * kHalf + kQBytes;
+  // followed by q of the group's heads, row-major: ratio * D * 2 bytes
+  static int wave_bytes(int ratio) { return 2 * kHalf + ratio * D * 2; }
 };
 
 // workspace layout: [batch][Hq][max_units][D + 2] floats (O[D] unnormalised, max, sum)
@@ -67,23 +67,12 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
   const int h0 = kvh * ratio;
   const int lh = lut_head(p.csr, h0, p.Hq, p.Hkv);
   if (rb >= p.csr.num_rows) return;
-  const int row0 = p.csr.ptr[lh * p.csr.ptr_sh + rb];
-  const int row1 = p.csr.ptr[lh * p.csr.ptr_sh + rb + 1];
+  // table reads go through the scalar unit (wave-uniform addresses, no vector-memory wait)
+  const int row0 = scalar_load(p.csr.ptr + lh * p.csr.ptr_sh + rb);
+  const int row1 = scalar_load(p.csr.ptr + lh * p.csr.ptr_sh + rb + 1);
   const int e0 = row0 + unit * unit_blocks;
   if (e0 >= row1) return;  // this row has fewer units
   const int e1 = min(e0 + unit_blocks, row1);
-
-  // q of the group's heads -> LDS (row min(m, ratio-1) feeds MFMA column m;
-  // columns >= ratio are duplicates whose results are never stored)
-  char *ks_ = smem, *vs_ = smem + S::kHalf, *qs_ = smem + 2 * S::kHalf;
-  {
-    const int hh = lane / CPR, ch = lane % CPR;  // 64 lanes cover 64 / CPR heads per pass
-    for (int h = hh; h < ratio; h += 64 / CPR) {
-      const T *qp = (const T *)p.q.ptr + sq.b * p.q.sb + (int64_t)(h0 + h) * p.q.sh + (int64_t)sq.q_start * p.q.st;
-      *reinterpret_cast<uint4 *>(qs_ + h * D * 2 + ch * 16) = *reinterpret_cast<const uint4 *>(qp + ch * 8);
-    }
-  }
-  const int q_read = (m < ratio ? m : ratio - 1) * D * 2 + g * 16;
   const int32_t *cols = p.csr.idx + lh * p.csr.idx_sh;
   const T *kbase = (const T *)p.k.ptr + sq.b * p.k.sb + kvh * p.k.sh + (int64_t)sq.k_start * p.k.st;
   const T *vbase = (const T *)p.v.ptr + sq.b * p.v.sb + kvh * p.v.sh + (int64_t)sq.k_start * p.v.st;
@@ -91,8 +80,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
   // half block hb of this unit = keys cols[e0 + hb/2] * 64 + 32 * (hb & 1) + [0, 32)
   constexpr int HCH = 32 * CPR / 64;  // 16-byte chunks per lane per half tile
   uint4 kreg[HCH], vreg[HCH];
-  auto prefetch = [&](int hb) {
-    const int col = cols[e0 + (hb >> 1)];
+  auto prefetch = [&](int hb, int col) {
     const int key0 = col * 64 + (hb & 1) * 32;
     if (col >= 0 && key0 + 32 <= sq.k_len) {  // whole half inside the sequence: no per-row guards
 #pragma unroll
@@ -115,6 +103,21 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
       }
     }
   };
+  // the first K/V request goes out before anything else touches memory
+  int col_cur = scalar_load(cols + e0);
+  prefetch(0, col_cur);
+
+  // q of the group's heads -> LDS (row min(m, ratio-1) feeds MFMA column m;
+  // columns >= ratio are duplicates whose results are never stored)
+  char *ks_ = smem, *vs_ = smem + S::kHalf, *qs_ = smem + 2 * S::kHalf;
+  {
+    const int hh = lane / CPR, ch = lane % CPR;  // 64 lanes cover 64 / CPR heads per pass
+    for (int h = hh; h < ratio; h += 64 / CPR) {
+      const T *qp = (const T *)p.q.ptr + sq.b * p.q.sb + (int64_t)(h0 + h) * p.q.sh + (int64_t)sq.q_start * p.q.st;
+      *reinterpret_cast<uint4 *>(qs_ + h * D * 2 + ch * 16) = *reinterpret_cast<const uint4 *>(qp + ch * 8);
+    }
+  }
+  const int q_read = (m < ratio ? m : ratio - 1) * D * 2 + g * 16;
 
   floatx16 oacc[DT];
 #pragma unroll
@@ -128,10 +131,11 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
   const int v_read = (4 * g + (i16 >> 2)) * S::kStride + (16 * dgrp + 4 * (i16 & 3)) * 2;
   const int nhalf = 2 * (e1 - e0);
 
-  prefetch(0);
   for (int hb = 0; hb < nhalf; ++hb) {
-    const int col = cols[e0 + (hb >> 1)];
+    const int col = col_cur;
     const int key0 = col * 64 + (hb & 1) * 32;
+    // table entry of the next half block (the next block after an odd half)
+    if ((hb & 1) && hb + 1 < nhalf) col_cur = scalar_load(cols + e0 + ((hb + 1) >> 1));
     // The tiles are private to this wave and LDS operations of one wave
     // execute in order, so the previous half block's reads are done; only the
     // compiler must not reorder across these points (a memory fence would
@@ -145,7 +149,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
       *reinterpret_cast<uint4 *>(vs_ + r * S::kStride + ch * 16) = vreg[c];
     }
     asm volatile("" ::: "memory");
-    if (hb + 1 < nhalf) prefetch(hb + 1);
+    if (hb + 1 < nhalf) prefetch(hb + 1, col_cur);
     if (col < 0 || key0 >= sq.k_len || (p.causal && key0 > pos)) continue;
 
     floatx16 sacc;
@@ -222,33 +226,62 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
   }
 }
 
+// Merge of the unit partials: one wave per (sequence, q head), lane l owns
+// dims {2l, 2l+1} (D = 128) or dim l (D = 64).  All loads of a row are issued
+// before the first use (units are few, a dependent load chain per unit would
+// make this small kernel latency-bound).
 template <typename T, int D>
-__global__ __launch_bounds__(D) void decode_combine_kernel(const FwdParams p, const float *ws, int unit_blocks,
-                                                           int max_units) {
-  const int h = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
+__global__ __launch_bounds__(64) void decode_combine_kernel(const FwdParams p, const float *ws, int unit_blocks,
+                                                            int max_units) {
+  constexpr int PER = D / 64;  // dims per lane
+  constexpr int MAXU = 8;      // units merged per pass
+  const int h = blockIdx.x, b = blockIdx.y, lane = threadIdx.x;
   const SeqInfo sq = load_seq(p.seqs, b, p.causal);
   if (sq.q_len <= 0) return;
   int units = 0;
   const int rb = sq.past / 64;
   if (sq.k_len > 0 && rb < p.csr.num_rows) {
     const int lh = lut_head(p.csr, h, p.Hq, p.Hkv);
-    const int n = p.csr.ptr[lh * p.csr.ptr_sh + rb + 1] - p.csr.ptr[lh * p.csr.ptr_sh + rb];
+    const int n = scalar_load(p.csr.ptr + lh * p.csr.ptr_sh + rb + 1) - scalar_load(p.csr.ptr + lh * p.csr.ptr_sh + rb);
     units = (n + unit_blocks - 1) / unit_blocks;
   }
   const float *src = ws + ((int64_t)b * p.Hq + h) * max_units * (D + 2);
-  float mmax = -INFINITY;
-  for (int s = 0; s < units; ++s) mmax = fmaxf(mmax, src[s * (D + 2) + D]);
-  const float muse = mmax == -INFINITY ? 0.f : mmax;
-  float o = 0.f, l = 0.f;
-  for (int s = 0; s < units; ++s) {
-    const float sc = fast_exp2(src[s * (D + 2) + D] - muse);
-    o += sc * src[s * (D + 2) + d];
-    l += sc * src[s * (D + 2) + D + 1];
+  float mmax = -INFINITY, l = 0.f, o[PER];
+#pragma unroll
+  for (int i = 0; i < PER; ++i) o[i] = 0.f;
+  for (int s0 = 0; s0 < units; s0 += MAXU) {
+    float mv[MAXU], lv[MAXU], ov[MAXU][PER];
+#pragma unroll
+    for (int s = 0; s < MAXU; ++s) {
+      const bool ok = s0 + s < units;
+      const float *row = src + (s0 + (ok ? s : 0)) * (D + 2);
+      mv[s] = ok ? row[D] : -INFINITY;
+      lv[s] = ok ? row[D + 1] : 0.f;
+#pragma unroll
+      for (int i = 0; i < PER; ++i) ov[s][i] = ok ? row[lane * PER + i] : 0.f;
+    }
+    float mnew = mmax;
+#pragma unroll
+    for (int s = 0; s < MAXU; ++s) mnew = fmaxf(mnew, mv[s]);
+    const float muse = mnew == -INFINITY ? 0.f : mnew;
+    const float alpha = fast_exp2(mmax - muse);  // exp2(-inf) = 0 on the first pass
+    l *= alpha;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) o[i] *= alpha;
+#pragma unroll
+    for (int s = 0; s < MAXU; ++s) {
+      const float sc = fast_exp2(mv[s] - muse);
+      l += sc * lv[s];
+#pragma unroll
+      for (int i = 0; i < PER; ++i) o[i] += sc * ov[s][i];
+    }
+    mmax = mnew;
   }
   const float inv = l > 0.f ? 1.f / l : 0.f;
   T *op = (T *)p.o.ptr + sq.b * p.o.sb + h * p.o.sh + (int64_t)sq.q_start * p.o.st;
-  op[d] = from_float<T>(o * inv);
-  if (p.lse.ptr && d == 0)
+#pragma unroll
+  for (int i = 0; i < PER; ++i) op[lane * PER + i] = from_float<T>(o[i] * inv);
+  if (p.lse.ptr && lane == 0)
     p.lse.ptr[sq.b * p.lse.sb + h * p.lse.sh + (int64_t)sq.q_start * p.lse.st] =
         l > 0.f ? (mmax + log2f(l)) * kLn2 : -INFINITY;
 }
@@ -275,13 +308,13 @@ size_t decode_workspace_bytes(const FwdParams &p) {
 
 template <typename T, int D>
 static int launch_decode_td(const FwdParams &p, float *ws, hipStream_t stream) {
-  constexpr int smem = DecSmem<D>::kWave;
+  const int smem = DecSmem<D>::wave_bytes(p.Hq / p.Hkv);
   const int unit_blocks = decode_unit_blocks(), max_units = decode_max_units(p);
   DK_REQUIRE(max_units <= 65535, "too many decode units");
   hipLaunchKernelGGL((decode_partial_kernel<T, D>), dim3(max_units, p.Hkv, p.seqs.batch), dim3(64), smem, stream,
                      p, ws, unit_blocks, max_units);
   DK_HIP_CHECK(hipGetLastError());
-  hipLaunchKernelGGL((decode_combine_kernel<T, D>), dim3(p.Hq, p.seqs.batch), dim3(D), 0, stream, p, ws,
+  hipLaunchKernelGGL((decode_combine_kernel<T, D>), dim3(p.Hq, p.seqs.batch), dim3(64), 0, stream, p, ws,
                      unit_blocks, max_units);
   DK_HIP_CHECK(hipGetLastError());
   return DK_OK;

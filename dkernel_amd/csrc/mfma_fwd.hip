@@ -27,6 +27,11 @@
 
 namespace dk {
 
+template <int V>
+struct Const {  // compile-time integer passed to a generic lambda
+  static constexpr int value = V;
+};
+
 template <int D>
 struct FwdSmem {  // one stage = K tile + V tile, swizzled row-major (mfma_common.h)
   static constexpr int kStage = 2 * Tile<D>::kBytes;
@@ -101,21 +106,28 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
 
   // loop-invariant LDS offsets of this lane's operand reads (row m of a 32-key tile, swizzled
   // chunk 2ks+g; transpose-read pairs of d-tile dt); tile / k-step row offsets are immediates
-  int rd[KS], tr[DT][2];
+  // (full pointers, and the stage is a compile-time constant of the loop body, so that stage,
+  // tile and k-step offsets all end up as instruction immediates)
+  const char *rd[KS], *tr[DT][2];
+  {
+    int tro[DT][2];
+    transposed_offsets<D>(lane, tro);
 #pragma unroll
-  for (int ks = 0; ks < KS; ++ks) rd[ks] = TL::off(m, 2 * ks + g);
-  transposed_offsets<D>(lane, tr);
+    for (int ks = 0; ks < KS; ++ks) rd[ks] = smem + TL::off(m, 2 * ks + g);
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) tr[dt][0] = smem + tro[dt][0], tr[dt][1] = smem + tro[dt][1];
+  }
 
   if (e0 < e1) issue(e0, 0);
-  for (int e = e0; e < e1; ++e) {
-    const int stage = (e - e0) & 1;
+  auto block_step = [&](int e, auto stage_tag) {
+    constexpr int stage = decltype(stage_tag)::value;
     const int col = cols[e];
     wait_tile_loads();
     __syncthreads();  // tile e is visible; every wave is done with the other stage
     if (e + 1 < e1) issue(e + 1, stage ^ 1);
     const int key0 = col * 64;
-    if (col < 0 || key0 >= sq.k_len || (p.causal && key0 > row0 + 31)) continue;  // nothing visible (wave-uniform)
-    const char *ks_ = smem + stage * S::kStage, *vs_ = ks_ + TL::kBytes;
+    if (col < 0 || key0 >= sq.k_len || (p.causal && key0 > row0 + 31)) return;  // nothing visible (wave-uniform)
+    constexpr int ks_ = stage * S::kStage, vs_ = ks_ + TL::kBytes;  // byte offsets of this stage's K and V tiles
 
     // S^T = K Q^T : two 32-key tiles.  Operand reads run one tile ahead of the
     // multiplies so that LDS latency is hidden behind the MFMA pipe.
@@ -131,15 +143,15 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
     {
       vec8 ka[2][KS];
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) ka[0][ks] = lds_read8<vec8>(ks_ + rd[ks]);
+      for (int ks = 0; ks < KS; ++ks) ka[0][ks] = lds_read8<vec8>(rd[ks] + ks_);
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) ka[1][ks] = lds_read8<vec8>(ks_ + 32 * TL::kRowBytes + rd[ks]);
+      for (int ks = 0; ks < KS; ++ks) ka[1][ks] = lds_read8<vec8>(rd[ks] + ks_ + 32 * TL::kRowBytes);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) sacc[0] = M::mma(ka[0][ks], qf[ks], sacc[0]);
       // first V^T operands do not depend on the softmax: fetch them behind the multiplies
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) va[0][dt] = lds_read_tr8<vec8>(vs_ + tr[dt][0], vs_ + tr[dt][1]);
+      for (int dt = 0; dt < DT; ++dt) va[0][dt] = lds_read_tr8<vec8>(tr[dt][0] + vs_, tr[dt][1] + vs_);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) sacc[1] = M::mma(ka[1][ks], qf[ks], sacc[1]);
@@ -198,13 +210,17 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
       for (int i = 0; i < 8; ++i) pf[i] = sacc[nt][t * 8 + i];
       const vec8 pb = M::pack(pf);
       if (step < 3) {
-        const char *vrow = vs_ + ((step + 1) * 16) * TL::kRowBytes;
+        const int vrow = vs_ + ((step + 1) * 16) * TL::kRowBytes;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) va[(step + 1) & 1][dt] = lds_read_tr8<vec8>(vrow + tr[dt][0], vrow + tr[dt][1]);
+        for (int dt = 0; dt < DT; ++dt) va[(step + 1) & 1][dt] = lds_read_tr8<vec8>(tr[dt][0] + vrow, tr[dt][1] + vrow);
       }
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) oacc[dt] = M::mma(va[step & 1][dt], pb, oacc[dt]);
     }
+  };
+  for (int e = e0; e < e1; e += 2) {
+    block_step(e, Const<0>{});
+    if (e + 1 < e1) block_step(e + 1, Const<1>{});
   }
 
   // l_run holds this lane's share of the row sum (keys with this lane's g)
@@ -238,11 +254,6 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
 // stages.  Same work split, grid and results as mfma_fwd_kernel.  Used for
 // one head per workgroup (G = 1, one wave per SIMD), where it measures faster.
 // ---------------------------------------------------------------------------
-template <int V>
-struct Const {
-  static constexpr int value = V;
-};
-
 template <typename T, int D, int G>
 __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 ? 1 : 2, 2))) void mfma_fwd_pipe_kernel(
     const FwdParams p, int tiles_y) {

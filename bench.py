@@ -26,6 +26,9 @@ sys.path.insert(0, ROOT)
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16, vendor figure
 HBM_PEAK_GBS = 8000.0            # MI355X HBM3E, vendor figure
+# HBM bytes per launch of the headline forward kernel, from rocprofv3 --pmc runs of this
+# file (FETCH_SIZE x 2.00 copy calibration = 231.4 MB, WRITE_SIZE = 136.3 MB); not measured live
+FWD_TRAFFIC_BYTES = 367.7e6
 BS, LOCAL, VERT, D = 64, 16, 8, 128
 
 
@@ -150,7 +153,9 @@ def main():
                    "active_blocks_per_batch": nnz, "flop_per_step": flops, "impl": args.impl},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_BF16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4),
-                     "traffic": None, "kernel_ms": round(ev_ms, 4)},
+                     "traffic": FWD_TRAFFIC_BYTES if args.impl == "auto" else None,
+                     "traffic_unit": "bytes per launch (rocprofv3 counters, separate run)",
+                     "algorithmic_bytes": 201.3e6 + 136.3e6, "kernel_ms": round(ev_ms, 4)},
     }
     del q, k, v
 

@@ -25,6 +25,17 @@
 
 namespace dk {
 
+template <int V>
+struct IntConst {  // compile-time integer passed to a generic lambda
+  static constexpr int value = V;
+};
+
+template <bool V>
+struct BoolConst {
+  static constexpr bool value = V;
+};
+
+
 // ---------------------------------------------------------------------------
 // dQ pass
 // ---------------------------------------------------------------------------
@@ -97,11 +108,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     kload.issue(reinterpret_cast<const char *>(kbase + (int64_t)key0 * p.k.st), 0, valid, ks);
     vload.issue(reinterpret_cast<const char *>(vbase + (int64_t)key0 * p.v.st), 0, valid, ks + TL::kBytes);
   };
-  // operand read offsets inside this wave's key half: row kh*32 + m, chunk 2ks+g swizzled
-  int rd[KS], tr[DT][2];
+  // operand read addresses inside this wave's key half (row kh*32 + m, chunk 2ks+g swizzled;
+  // transpose-read pairs) for a tile at offset 0: full pointers, and the stage is a compile-time
+  // constant of the loop body, so that stage and k-step offsets are instruction immediates
+  const char *rd[KS], *tr[DT][2];
+  {
+    int tro[DT][2];
+    transposed_offsets<D>(lane, tro);
 #pragma unroll
-  for (int ks = 0; ks < KS; ++ks) rd[ks] = TL::off(kh * 32 + m, 2 * ks + g);
-  transposed_offsets<D>(lane, tr);
+    for (int ks = 0; ks < KS; ++ks) rd[ks] = smem + TL::off(kh * 32 + m, 2 * ks + g);
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+      tr[dt][0] = smem + kh * 32 * TL::kRowBytes + tro[dt][0], tr[dt][1] = smem + kh * 32 * TL::kRowBytes + tro[dt][1];
+  }
 
   floatx16 acc[DT];
 #pragma unroll
@@ -110,15 +129,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     for (int r = 0; r < 16; ++r) acc[dt][r] = 0.f;
 
   if (e0 < e1) issue(e0, 0);
-  for (int e = e0; e < e1; ++e) {
-    const int stage = (e - e0) & 1;
+  auto block_step = [&](int e, auto stage_tag) {
+    constexpr int stage = decltype(stage_tag)::value;
     const int col = cols[e];
     wait_tile_loads();
     __syncthreads();  // tile e is visible; every wave is done with the other stage
     if (e + 1 < e1) issue(e + 1, stage ^ 1);
     const int key0 = col * 64 + kh * 32;  // first key of this wave's half
-    if (col < 0 || key0 >= sq.k_len || (p.causal && key0 > row0 + 31)) continue;
-    const char *ks_ = smem + stage * STAGE, *vs_ = ks_ + TL::kBytes;
+    if (col < 0 || key0 >= sq.k_len || (p.causal && key0 > row0 + 31)) return;
+    constexpr int ks_ = stage * STAGE, vs_ = ks_ + TL::kBytes;  // byte offsets of this stage's K and V tiles
 
     floatx16 s, dp;
 #pragma unroll
@@ -129,7 +148,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     for (int half = 0; half < 2; ++half) {
       vec8 ka[KS / 2];
 #pragma unroll
-      for (int i = 0; i < KS / 2; ++i) ka[i] = lds_read8<vec8>(ks_ + rd[half * (KS / 2) + i]);
+      for (int i = 0; i < KS / 2; ++i) ka[i] = lds_read8<vec8>(rd[half * (KS / 2) + i] + ks_);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < KS / 2; ++i) s = M::mma(ka[i], qf[half * (KS / 2) + i], s);
@@ -138,28 +157,29 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     for (int half = 0; half < 2; ++half) {
       vec8 va[KS / 2];
 #pragma unroll
-      for (int i = 0; i < KS / 2; ++i) va[i] = lds_read8<vec8>(vs_ + rd[half * (KS / 2) + i]);
+      for (int i = 0; i < KS / 2; ++i) va[i] = lds_read8<vec8>(rd[half * (KS / 2) + i] + vs_);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < KS / 2; ++i) dp = M::mma(va[i], dof[half * (KS / 2) + i], dp);
     }
     // K^T operands of the dQ product do not depend on dS: fetch them now
-    const char *krow = ks_ + kh * 32 * TL::kRowBytes;
     vec8 kt[DT];
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) kt[dt] = lds_read_tr8<vec8>(krow + tr[dt][0], krow + tr[dt][1]);
+    for (int dt = 0; dt < DT; ++dt) kt[dt] = lds_read_tr8<vec8>(tr[dt][0] + ks_, tr[dt][1] + ks_);
 
     const bool need_mask = (key0 + 31 >= sq.k_len) || (p.causal && key0 + 31 > row0);
     const int lim = p.causal ? min(pos, sq.k_len - 1) : sq.k_len - 1;  // last visible key of this row
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      float pr = fast_exp2(fmaf(s[r], p.scale_log2, -lse2));
-      if (need_mask) {
+    for (int r = 0; r < 16; ++r) s[r] = fast_exp2(fmaf(s[r], p.scale_log2, -lse2));
+    if (need_mask) {  // wave-uniform: only the diagonal block and the last, partial one pay for masks
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
         const int key = key0 + (r >> 2) * 8 + g * 4 + (r & 3);
-        pr = key > lim ? 0.f : pr;
+        s[r] = key > lim ? 0.f : s[r];
       }
-      s[r] = pr * (dp[r] - delta);  // dS^T without sm_scale (applied once at the end)
     }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s[r] *= dp[r] - delta;  // dS^T without sm_scale (applied once at the end)
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       float f[8];
@@ -170,9 +190,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       for (int dt = 0; dt < DT; ++dt) {
         acc[dt] = M::mma(kt[dt], dsb, acc[dt]);
         if (t == 0)  // refill with the second k-step's operand as soon as the register is free
-          kt[dt] = lds_read_tr8<vec8>(krow + 16 * TL::kRowBytes + tr[dt][0], krow + 16 * TL::kRowBytes + tr[dt][1]);
+          kt[dt] = lds_read_tr8<vec8>(tr[dt][0] + ks_ + 16 * TL::kRowBytes, tr[dt][1] + ks_ + 16 * TL::kRowBytes);
       }
     }
+  };
+  for (int e = e0; e < e1; e += 2) {
+    block_step(e, IntConst<0>{});
+    if (e + 1 < e1) block_step(e + 1, IntConst<1>{});
   }
 
   // sum the two key halves: waves with kh = 1 hand their partial to kh = 0
@@ -216,11 +240,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 // barrier per block is enough: Q tiles and the lse / delta vectors live one
 // iteration longer than dO tiles (rings of 4 and 3 stages), and tile loads run
 // two blocks ahead.
-template <bool V>
-struct BoolConst {
-  static constexpr bool value = V;
-};
-
 template <int D>
 struct DkdvSmem {
   using TL = Tile<D>;

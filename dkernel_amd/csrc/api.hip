@@ -10,7 +10,7 @@
 namespace dk {
 
 int launch_generic_fwd(const FwdParams &p, int dtype, hipStream_t stream);
-int launch_generic_bwd(const BwdParams &p, int dtype, hipStream_t stream, bool delta_only);
+int launch_generic_bwd(const BwdParams &p, int dtype, hipStream_t stream);
 bool mfma_fwd_supported(const FwdParams &p, int dtype);
 int launch_mfma_fwd(const FwdParams &p, int dtype, hipStream_t stream);
 bool mfma_bwd_supported(const BwdParams &p, int dtype);
@@ -172,15 +172,13 @@ int dk_bwd(const dk_bwd_args *a) {
   hipStream_t stream = (hipStream_t)a->stream;
   if (a->impl != DK_IMPL_GENERIC) {
     if (mfma_bwd_supported(p, a->dtype)) {
-      rc = launch_generic_bwd(p, a->dtype, stream, /*delta_only=*/true);
-      if (rc) return rc;
       return launch_mfma_bwd(p, a->dtype, stream);
     }
     if (a->impl == DK_IMPL_MFMA)
       return fail(DK_ERR_UNSUPPORTED, "no MFMA backward kernel for dtype %d, head_dim %d, tiles (%d, %d)",
                   a->dtype, p.D, p.csr.block_rows, p.csr.block_cols);
   }
-  return launch_generic_bwd(p, a->dtype, stream, /*delta_only=*/false);
+  return launch_generic_bwd(p, a->dtype, stream);
 }
 
 }  // extern "C"

@@ -309,13 +309,12 @@ __global__ __launch_bounds__(256) void generic_dkdv_kernel(const BwdParams p) {
 }
 
 template <typename T, int DPAD>
-static int launch_bwd_td(const BwdParams &p, hipStream_t stream, bool delta_only) {
+static int launch_bwd_td(const BwdParams &p, hipStream_t stream) {
   constexpr int R = 256 / (DPAD / 32);
   const SeqView &s = p.seqs;
   hipLaunchKernelGGL((generic_delta_kernel<T, DPAD>), dim3(cdiv(s.max_q_len, R), p.Hq, s.batch), dim3(256), 0,
                      stream, p);
   DK_HIP_CHECK(hipGetLastError());
-  if (delta_only) return DK_OK;
   {
     const int BM = p.csr.block_rows;
     const int rows_wg = BM < R ? BM : R;
@@ -336,19 +335,17 @@ static int launch_bwd_td(const BwdParams &p, hipStream_t stream, bool delta_only
 }
 
 template <typename T>
-static int launch_bwd_t(const BwdParams &p, hipStream_t stream, bool delta_only) {
-  if (p.D <= 64) return launch_bwd_td<T, 64>(p, stream, delta_only);
-  if (p.D <= 128) return launch_bwd_td<T, 128>(p, stream, delta_only);
-  return launch_bwd_td<T, 256>(p, stream, delta_only);
+static int launch_bwd_t(const BwdParams &p, hipStream_t stream) {
+  if (p.D <= 64) return launch_bwd_td<T, 64>(p, stream);
+  if (p.D <= 128) return launch_bwd_td<T, 128>(p, stream);
+  return launch_bwd_td<T, 256>(p, stream);
 }
 
-// delta_only: just the preprocess pass (the MFMA path runs its own dQ and
-// dK/dV kernels afterwards).
-int launch_generic_bwd(const BwdParams &p, int dtype, hipStream_t stream, bool delta_only) {
+int launch_generic_bwd(const BwdParams &p, int dtype, hipStream_t stream) {
   switch (dtype) {
-    case DK_BF16: return launch_bwd_t<bf16_t>(p, stream, delta_only);
-    case DK_F16: return launch_bwd_t<f16_t>(p, stream, delta_only);
-    case DK_F32: return launch_bwd_t<float>(p, stream, delta_only);
+    case DK_BF16: return launch_bwd_t<bf16_t>(p, stream);
+    case DK_F16: return launch_bwd_t<f16_t>(p, stream);
+    case DK_F32: return launch_bwd_t<float>(p, stream);
   }
   return fail(DK_ERR_UNSUPPORTED, "unknown dtype %d", dtype);
 }

@@ -65,33 +65,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int qi = pos - sq.past;
   const bool row_ok = qi >= 0 && qi < sq.q_len;
 
-  vec8 qf[KS], dof[KS];
-  float lse2 = INFINITY, delta = 0.f;
-  {
-    const T *qp = (const T *)p.q.ptr + sq.b * p.q.sb + h * p.q.sh + (int64_t)qi * p.q.st;
-    const T *dop = (const T *)p.dout.ptr + sq.b * p.dout.sb + h * p.dout.sh + (int64_t)qi * p.dout.st;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      uint4 a = make_uint4(0, 0, 0, 0), b = a;
-      if (row_ok) {
-        a = *reinterpret_cast<const uint4 *>(qp + ks * 16 + g * 8);
-        b = *reinterpret_cast<const uint4 *>(dop + ks * 16 + g * 8);
-      }
-      qf[ks] = as_vec8<vec8>(a);
-      dof[ks] = as_vec8<vec8>(b);
-    }
-    if (row_ok) {
-      const float l = p.lse.ptr[sq.b * p.lse.sb + h * p.lse.sh + (int64_t)qi * p.lse.st];
-      lse2 = l == -INFINITY ? INFINITY : l * kLog2e;
-      delta = p.delta[((int64_t)sq.b * p.Hq + h) * p.seqs.max_q_len + qi];
-    }
-  }
-
   const int lh = lut_head(p.csr, h, p.Hq, p.Hkv);
+  // table reads go through the scalar unit: a vector load would have to be waited for with
+  // vmcnt(0), i.e. together with every tile copy in flight
   int e0 = 0, e1 = 0;
   if (rb < p.csr.num_rows) {
-    e0 = p.csr.ptr[lh * p.csr.ptr_sh + rb];
-    e1 = p.csr.ptr[lh * p.csr.ptr_sh + rb + 1];
+    e0 = scalar_load(p.csr.ptr + lh * p.csr.ptr_sh + rb);
+    e1 = scalar_load(p.csr.ptr + lh * p.csr.ptr_sh + rb + 1);
   }
   const int32_t *cols = p.csr.idx + lh * p.csr.idx_sh;
   const T *kbase = (const T *)p.k.ptr + sq.b * p.k.sb + kvh * p.k.sh;
@@ -101,7 +81,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   kload.init(tid, p.k.st);
   vload.init(tid, p.v.st);
   auto issue = [&](int e, int stage) {  // asynchronous copy of block e's K and V tiles into `stage`
-    const int col = cols[e];
+    const int col = scalar_load(cols + e);
     const int key0 = col * 64;
     const int valid = col < 0 ? 0 : sq.k_len - key0;
     char *ks = smem + stage * STAGE;
@@ -128,10 +108,40 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[dt][r] = 0.f;
 
-  if (e0 < e1) issue(e0, 0);
+  if (e0 < e1) issue(e0, 0);  // the first tiles are on their way while the row data is fetched
+
+  // Q and dO fragments of this lane's row, its lse, and delta = rowsum(O * dO) - dLSE, which
+  // this kernel computes itself and also leaves in p.delta for the dK/dV pass that follows
+  vec8 qf[KS], dof[KS];
+  float lse2 = INFINITY, delta = 0.f;
+  {
+    const T *qp = (const T *)p.q.ptr + sq.b * p.q.sb + h * p.q.sh + (int64_t)qi * p.q.st;
+    const T *dop = (const T *)p.dout.ptr + sq.b * p.dout.sb + h * p.dout.sh + (int64_t)qi * p.dout.st;
+    const T *op = (const T *)p.o.ptr + sq.b * p.o.sb + h * p.o.sh + (int64_t)qi * p.o.st;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      uint4 a = make_uint4(0, 0, 0, 0), b = a, c = a;
+      if (row_ok) {
+        a = *reinterpret_cast<const uint4 *>(qp + ks * 16 + g * 8);
+        b = *reinterpret_cast<const uint4 *>(dop + ks * 16 + g * 8);
+        c = *reinterpret_cast<const uint4 *>(op + ks * 16 + g * 8);
+      }
+      qf[ks] = as_vec8<vec8>(a);
+      dof[ks] = as_vec8<vec8>(b);
+      delta = dot8<T>(c, b, delta);
+    }
+    delta += xor32(delta);  // the two half-waves hold the two halves of the row's head dims
+    if (row_ok) {
+      const float l = p.lse.ptr[sq.b * p.lse.sb + h * p.lse.sh + (int64_t)qi * p.lse.st];
+      lse2 = l == -INFINITY ? INFINITY : l * kLog2e;
+      if (p.dlse.ptr) delta -= p.dlse.ptr[sq.b * p.dlse.sb + h * p.dlse.sh + (int64_t)qi * p.dlse.st];
+      if (kh == 0 && g == 0) p.delta[((int64_t)sq.b * p.Hq + h) * p.seqs.max_q_len + qi] = delta;
+    }
+  }
+
   auto block_step = [&](int e, auto stage_tag) {
     constexpr int stage = decltype(stage_tag)::value;
-    const int col = cols[e];
+    const int col = scalar_load(cols + e);
     wait_tile_loads();
     __syncthreads();  // tile e is visible; every wave is done with the other stage
     if (e + 1 < e1) issue(e + 1, stage ^ 1);
@@ -556,9 +566,10 @@ static int launch_bwd_td(const BwdParams &p, hipStream_t stream) {
   const int tiles = (past + s.max_q_len - 1) / 64 - past / 64 + 1;
   const int cblocks = cdiv(s.max_k_len, 64);
   DK_REQUIRE(tiles <= 65535 && cblocks <= 65535, "sequence too long for one launch");
-  hipLaunchKernelGGL((mfma_dkdv_kernel<T, D>), dim3(p.Hkv, cblocks, s.batch), dim3(512), smem_dkdv, stream, p);
-  DK_HIP_CHECK(hipGetLastError());
+  // dQ first: it also writes delta, which the dK/dV pass reads
   hipLaunchKernelGGL((mfma_dq_kernel<T, D>), dim3(p.Hq, tiles, s.batch), dim3(256), smem_dq, stream, p, tiles);
+  DK_HIP_CHECK(hipGetLastError());
+  hipLaunchKernelGGL((mfma_dkdv_kernel<T, D>), dim3(p.Hkv, cblocks, s.batch), dim3(512), smem_dkdv, stream, p);
   DK_HIP_CHECK(hipGetLastError());
   return DK_OK;
 }

@@ -60,6 +60,26 @@ struct Mma<f16_t> {
   }
 };
 
+// acc + dot product of two 16-byte groups of eight 16-bit values (exact fp32 products)
+template <typename T>
+__device__ __forceinline__ float dot8(uint4 a, uint4 b, float acc);
+template <>
+__device__ __forceinline__ float dot8<bf16_t>(uint4 a, uint4 b, float acc) {
+  typedef __bf16 v2 __attribute__((ext_vector_type(2)));
+  acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(v2, a.x), __builtin_bit_cast(v2, b.x), acc, false);
+  acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(v2, a.y), __builtin_bit_cast(v2, b.y), acc, false);
+  acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(v2, a.z), __builtin_bit_cast(v2, b.z), acc, false);
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(v2, a.w), __builtin_bit_cast(v2, b.w), acc, false);
+}
+template <>
+__device__ __forceinline__ float dot8<f16_t>(uint4 a, uint4 b, float acc) {
+  typedef _Float16 v2 __attribute__((ext_vector_type(2)));
+  acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(v2, a.x), __builtin_bit_cast(v2, b.x), acc, false);
+  acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(v2, a.y), __builtin_bit_cast(v2, b.y), acc, false);
+  acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(v2, a.z), __builtin_bit_cast(v2, b.z), acc, false);
+  return __builtin_amdgcn_fdot2(__builtin_bit_cast(v2, a.w), __builtin_bit_cast(v2, b.w), acc, false);
+}
+
 template <typename V>
 __device__ __forceinline__ V as_vec8(uint4 w) {
   return __builtin_bit_cast(V, w);

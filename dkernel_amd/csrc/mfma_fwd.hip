@@ -76,9 +76,9 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
 
   const int lh = lut_head(p.csr, blockIdx.x * G, p.Hq, p.Hkv);
   int e0 = 0, e1 = 0;
-  if (rb < p.csr.num_rows) {
-    e0 = p.csr.ptr[lh * p.csr.ptr_sh + rb];
-    e1 = p.csr.ptr[lh * p.csr.ptr_sh + rb + 1];
+  if (rb < p.csr.num_rows) {  // table reads go through the scalar unit (no vector-memory wait)
+    e0 = scalar_load(p.csr.ptr + lh * p.csr.ptr_sh + rb);
+    e1 = scalar_load(p.csr.ptr + lh * p.csr.ptr_sh + rb + 1);
   }
   const int32_t *cols = p.csr.idx + lh * p.csr.idx_sh;
   const T *kbase = (const T *)p.k.ptr + sq.b * p.k.sb + kvh * p.k.sh + (int64_t)sq.k_start * p.k.st;
@@ -89,7 +89,7 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
   kload.init(tid, p.k.st);
   vload.init(tid, p.v.st);
   auto issue = [&](int e, int stage) {
-    const int col = cols[e];
+    const int col = scalar_load(cols + e);
     const int key0 = col * 64;
     const int valid = col < 0 ? 0 : sq.k_len - key0;
     char *ks = smem + stage * S::kStage;
@@ -121,7 +121,7 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
   if (e0 < e1) issue(e0, 0);
   auto block_step = [&](int e, auto stage_tag) {
     constexpr int stage = decltype(stage_tag)::value;
-    const int col = cols[e];
+    const int col = scalar_load(cols + e);
     wait_tile_loads();
     __syncthreads();  // tile e is visible; every wave is done with the other stage
     if (e + 1 < e1) issue(e + 1, stage ^ 1);
@@ -304,7 +304,7 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
   TileLoader<D, NT> kload, vload;
   kload.init(tid, p.k.st);
   vload.init(tid, p.v.st);
-  // table entries are read well before they are needed and never between a tile load and
+  // table entries are read well before they are needed and never between a tile request and
   // its wait (a vector load there would make the wait cover the tile just requested)
   auto col_at = [&](int j) { return __builtin_amdgcn_readfirstlane(j < n ? cols[j] : 0); };
   auto issue_k = [&](int stage, int col) {

@@ -3,20 +3,24 @@
 //
 //   dQ pass    (CSR rows)    workgroup = 64 q rows x one q head, 4 waves = 2 row
 //              halves x 2 key halves (2 waves per SIMD; the key halves are
-//              summed through LDS at the end).  Per listed K/V block: S^T = K Q^T, dP^T = V dO^T (lane =
-//              q row, registers = keys, so lse / delta are per-lane scalars),
-//              dS^T = P^T (dP^T - delta), dQ^T += K^T dS^T with dS^T fed from
-//              registers as the B operand and K^T from LDS transpose reads.
+//              summed through LDS at the end).  Per listed K/V block:
+//              S^T = K Q^T, dP^T = V dO^T (lane = q row, registers = keys, so
+//              lse / delta are per-lane scalars), dS^T = P^T (dP^T - delta),
+//              dQ^T += K^T dS^T with dS^T fed from registers as the B operand
+//              and K^T from LDS transpose reads.  The pass also computes
+//              delta = rowsum(O * dO) - dLSE of its rows and leaves it in
+//              memory for the dK/dV pass, which therefore runs second.
 //   dK/dV pass (CSC columns) workgroup = 64 keys x one kv head (the q heads of
-//              a GQA group are looped inside), 4 waves = 2 key halves x 2 q-row
-//              halves.  K and V fragments stay in registers; per listed q
-//              block: S = Q K^T, dP = dO V^T (lane = key, registers = q rows),
-//              dV^T += dO^T P, dK^T += Q^T dS with P / dS from registers and
-//              dO^T / Q^T from LDS transpose reads.  The two q-row halves are
-//              summed through LDS at the end.
+//              a GQA group are looped inside), 8 waves: every 32 x 32 quadrant
+//              (q-row half x key half) has an S wave (S = Q K^T, P, dV^T +=
+//              dO^T P; K fragments in registers) and a dP wave (dP = dO V^T,
+//              dS = P (dP - delta), dK^T += Q^T dS; V fragments in registers).
+//              P / dS feed the second products from registers, dO^T / Q^T
+//              come from LDS transpose reads.  The two q-row halves are summed
+//              through LDS at the end.
 //
-// Tiles are copied HBM -> LDS asynchronously (no staging registers), double
-// buffered, in the swizzled row-major layout of mfma_common.h.
+// Tiles are copied HBM -> LDS asynchronously (LDS DMA, no staging registers)
+// into rings of stages, in the swizzled row-major layout of mfma_common.h.
 #include <climits>
 
 #include "common.h"
@@ -80,8 +84,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   TileLoader<D, NT> kload, vload;
   kload.init(tid, p.k.st);
   vload.init(tid, p.v.st);
-  auto issue = [&](int e, int stage) {  // asynchronous copy of block e's K and V tiles into `stage`
-    const int col = scalar_load(cols + e);
+  auto issue = [&](int col, int stage) {  // asynchronous copy of K/V block `col` into `stage`
     const int key0 = col * 64;
     const int valid = col < 0 ? 0 : sq.k_len - key0;
     char *ks = smem + stage * STAGE;
@@ -108,7 +111,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[dt][r] = 0.f;
 
-  if (e0 < e1) issue(e0, 0);  // the first tiles are on their way while the row data is fetched
+  // Table entries: block e in col_cur (scalar register); block e + 1 is requested one block
+  // early as a vector load (col_pending) and first used behind the next tile wait, so that no
+  // table read ever stalls the loop.
+  int col_cur = e0 < e1 ? scalar_load(cols + e0) : 0;
+  int col_pending = e0 + 1 < e1 ? cols[e0 + 1] : 0;
+  if (e0 < e1) issue(col_cur, 0);  // the first tiles are on their way while the row data is fetched
 
   // Q and dO fragments of this lane's row, its lse, and delta = rowsum(O * dO) - dLSE, which
   // this kernel computes itself and also leaves in p.delta for the dK/dV pass that follows
@@ -141,10 +149,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
   auto block_step = [&](int e, auto stage_tag) {
     constexpr int stage = decltype(stage_tag)::value;
-    const int col = scalar_load(cols + e);
+    const int col = col_cur;
     wait_tile_loads();
     __syncthreads();  // tile e is visible; every wave is done with the other stage
-    if (e + 1 < e1) issue(e + 1, stage ^ 1);
+    const int col_next = __builtin_amdgcn_readfirstlane(col_pending);  // landed before the tile did
+    if (e + 2 < e1) col_pending = cols[e + 2];
+    if (e + 1 < e1) issue(col_next, stage ^ 1);
+    col_cur = col_next;
     const int key0 = col * 64 + kh * 32;  // first key of this wave's half
     if (col < 0 || key0 >= sq.k_len || (p.causal && key0 > row0 + 31)) return;
     constexpr int ks_ = stage * STAGE, vs_ = ks_ + TL::kBytes;  // byte offsets of this stage's K and V tiles

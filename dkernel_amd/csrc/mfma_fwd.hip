@@ -88,8 +88,7 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
   TileLoader<D, NT> kload, vload;
   kload.init(tid, p.k.st);
   vload.init(tid, p.v.st);
-  auto issue = [&](int e, int stage) {
-    const int col = scalar_load(cols + e);
+  auto issue = [&](int col, int stage) {
     const int key0 = col * 64;
     const int valid = col < 0 ? 0 : sq.k_len - key0;
     char *ks = smem + stage * S::kStage;
@@ -118,13 +117,21 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
     for (int dt = 0; dt < DT; ++dt) tr[dt][0] = smem + tro[dt][0], tr[dt][1] = smem + tro[dt][1];
   }
 
-  if (e0 < e1) issue(e0, 0);
+  // Table entries: block e in col_cur (scalar register); block e + 1 is requested one block
+  // early as a vector load (col_pending) and first used behind the next tile wait, so that no
+  // table read ever stalls the loop.
+  int col_cur = e0 < e1 ? scalar_load(cols + e0) : 0;
+  int col_pending = e0 + 1 < e1 ? cols[e0 + 1] : 0;
+  if (e0 < e1) issue(col_cur, 0);
   auto block_step = [&](int e, auto stage_tag) {
     constexpr int stage = decltype(stage_tag)::value;
-    const int col = scalar_load(cols + e);
+    const int col = col_cur;
     wait_tile_loads();
     __syncthreads();  // tile e is visible; every wave is done with the other stage
-    if (e + 1 < e1) issue(e + 1, stage ^ 1);
+    const int col_next = __builtin_amdgcn_readfirstlane(col_pending);  // landed before the tile did
+    if (e + 2 < e1) col_pending = cols[e + 2];
+    if (e + 1 < e1) issue(col_next, stage ^ 1);
+    col_cur = col_next;
     const int key0 = col * 64;
     if (col < 0 || key0 >= sq.k_len || (p.causal && key0 > row0 + 31)) return;  // nothing visible (wave-uniform)
     constexpr int ks_ = stage * S::kStage, vs_ = ks_ + TL::kBytes;  // byte offsets of this stage's K and V tiles

@@ -68,8 +68,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
   const int lh = lut_head(p.csr, h0, p.Hq, p.Hkv);
   if (rb >= p.csr.num_rows) return;
   // table reads go through the scalar unit (wave-uniform addresses, no vector-memory wait)
-  const int row0 = scalar_load(p.csr.ptr + lh * p.csr.ptr_sh + rb);
-  const int row1 = scalar_load(p.csr.ptr + lh * p.csr.ptr_sh + rb + 1);
+  int row0, row1;
+  scalar_load2(p.csr.ptr + lh * p.csr.ptr_sh + rb, p.csr.ptr + lh * p.csr.ptr_sh + rb + 1, row0, row1);
   const int e0 = row0 + unit * unit_blocks;
   if (e0 >= row1) return;  // this row has fewer units
   const int e1 = min(e0 + unit_blocks, row1);

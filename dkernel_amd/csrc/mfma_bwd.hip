@@ -69,13 +69,36 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int qi = pos - sq.past;
   const bool row_ok = qi >= 0 && qi < sq.q_len;
 
+  // Row data of this lane (Q, dO, O fragments, lse, dLSE) is requested before anything else, so
+  // that its round trip overlaps with the table reads and the first tile request; it is used
+  // only after that request has gone out.
+  uint4 qraw[KS], doraw[KS], oraw[KS];
+  float lse_raw = -INFINITY, dlse_raw = 0.f;
+  {
+    const T *qp = (const T *)p.q.ptr + sq.b * p.q.sb + h * p.q.sh + (int64_t)qi * p.q.st;
+    const T *dop = (const T *)p.dout.ptr + sq.b * p.dout.sb + h * p.dout.sh + (int64_t)qi * p.dout.st;
+    const T *op = (const T *)p.o.ptr + sq.b * p.o.sb + h * p.o.sh + (int64_t)qi * p.o.st;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      qraw[ks] = doraw[ks] = oraw[ks] = make_uint4(0, 0, 0, 0);
+      if (row_ok) {
+        qraw[ks] = *reinterpret_cast<const uint4 *>(qp + ks * 16 + g * 8);
+        doraw[ks] = *reinterpret_cast<const uint4 *>(dop + ks * 16 + g * 8);
+        oraw[ks] = *reinterpret_cast<const uint4 *>(op + ks * 16 + g * 8);
+      }
+    }
+    if (row_ok) {
+      lse_raw = p.lse.ptr[sq.b * p.lse.sb + h * p.lse.sh + (int64_t)qi * p.lse.st];
+      if (p.dlse.ptr) dlse_raw = p.dlse.ptr[sq.b * p.dlse.sb + h * p.dlse.sh + (int64_t)qi * p.dlse.st];
+    }
+  }
+
   const int lh = lut_head(p.csr, h, p.Hq, p.Hkv);
   // table reads go through the scalar unit: a vector load would have to be waited for with
   // vmcnt(0), i.e. together with every tile copy in flight
   int e0 = 0, e1 = 0;
   if (rb < p.csr.num_rows) {
-    e0 = scalar_load(p.csr.ptr + lh * p.csr.ptr_sh + rb);
-    e1 = scalar_load(p.csr.ptr + lh * p.csr.ptr_sh + rb + 1);
+    scalar_load2(p.csr.ptr + lh * p.csr.ptr_sh + rb, p.csr.ptr + lh * p.csr.ptr_sh + rb + 1, e0, e1);
   }
   const int32_t *cols = p.csr.idx + lh * p.csr.idx_sh;
   const T *kbase = (const T *)p.k.ptr + sq.b * p.k.sb + kvh * p.k.sh;
@@ -118,33 +141,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   int col_pending = e0 + 1 < e1 ? cols[e0 + 1] : 0;
   if (e0 < e1) issue(col_cur, 0);  // the first tiles are on their way while the row data is fetched
 
-  // Q and dO fragments of this lane's row, its lse, and delta = rowsum(O * dO) - dLSE, which
-  // this kernel computes itself and also leaves in p.delta for the dK/dV pass that follows
+  // Q and dO fragments, lse in the log2 domain, and delta = rowsum(O * dO) - dLSE, which this
+  // kernel computes itself and also leaves in p.delta for the dK/dV pass that follows
   vec8 qf[KS], dof[KS];
   float lse2 = INFINITY, delta = 0.f;
-  {
-    const T *qp = (const T *)p.q.ptr + sq.b * p.q.sb + h * p.q.sh + (int64_t)qi * p.q.st;
-    const T *dop = (const T *)p.dout.ptr + sq.b * p.dout.sb + h * p.dout.sh + (int64_t)qi * p.dout.st;
-    const T *op = (const T *)p.o.ptr + sq.b * p.o.sb + h * p.o.sh + (int64_t)qi * p.o.st;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      uint4 a = make_uint4(0, 0, 0, 0), b = a, c = a;
-      if (row_ok) {
-        a = *reinterpret_cast<const uint4 *>(qp + ks * 16 + g * 8);
-        b = *reinterpret_cast<const uint4 *>(dop + ks * 16 + g * 8);
-        c = *reinterpret_cast<const uint4 *>(op + ks * 16 + g * 8);
-      }
-      qf[ks] = as_vec8<vec8>(a);
-      dof[ks] = as_vec8<vec8>(b);
-      delta = dot8<T>(c, b, delta);
-    }
-    delta += xor32(delta);  // the two half-waves hold the two halves of the row's head dims
-    if (row_ok) {
-      const float l = p.lse.ptr[sq.b * p.lse.sb + h * p.lse.sh + (int64_t)qi * p.lse.st];
-      lse2 = l == -INFINITY ? INFINITY : l * kLog2e;
-      if (p.dlse.ptr) delta -= p.dlse.ptr[sq.b * p.dlse.sb + h * p.dlse.sh + (int64_t)qi * p.dlse.st];
-      if (kh == 0 && g == 0) p.delta[((int64_t)sq.b * p.Hq + h) * p.seqs.max_q_len + qi] = delta;
-    }
+  for (int ks = 0; ks < KS; ++ks) {
+    qf[ks] = as_vec8<vec8>(qraw[ks]);
+    dof[ks] = as_vec8<vec8>(doraw[ks]);
+    delta = dot8<T>(oraw[ks], doraw[ks], delta);
+  }
+  delta += xor32(delta);  // the two half-waves hold the two halves of the row's head dims
+  if (row_ok) {
+    lse2 = lse_raw == -INFINITY ? INFINITY : lse_raw * kLog2e;
+    delta -= dlse_raw;
+    if (kh == 0 && g == 0) p.delta[((int64_t)sq.b * p.Hq + h) * p.seqs.max_q_len + qi] = delta;
   }
 
   auto block_step = [&](int e, auto stage_tag) {
@@ -329,11 +340,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int h = kvh * ratio + gq;
     const int lh = lut_head(p.csc, h, p.Hq, p.Hkv);
     int e0 = 0, e1 = 0;
-    if (cb < p.csc.num_rows) {
-      e0 = p.csc.ptr[lh * p.csc.ptr_sh + cb];
-      e1 = p.csc.ptr[lh * p.csc.ptr_sh + cb + 1];
-    }
-    const int nblk = __builtin_amdgcn_readfirstlane(e1 - e0);
+    if (cb < p.csc.num_rows)
+      scalar_load2(p.csc.ptr + lh * p.csc.ptr_sh + cb, p.csc.ptr + lh * p.csc.ptr_sh + cb + 1, e0, e1);
+    const int nblk = e1 - e0;
     const int32_t *rows = p.csc.idx + lh * p.csc.idx_sh + e0;
     const T *qbase = (const T *)p.q.ptr + sq.b * p.q.sb + h * p.q.sh;
     const T *dobase = (const T *)p.dout.ptr + sq.b * p.dout.sb + h * p.dout.sh;
@@ -344,8 +353,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // its rows (even waves copy lse, odd waves delta; they all write the same values, so that
     // every wave issues the same number of load instructions).  Returns false when rows had
     // to be zero-filled, i.e. when the per-wave load count is not LPT.
-    auto issue = [&](int t, int qstage, int dostage) -> bool {
-      const int rbq = scalar_load(rows + t);
+    auto issue = [&](int rbq, int qstage, int dostage) -> bool {
       const int qi0 = rbq * 64 - sq.past;  // query index of the tile's first row
       // rows before the first query (qi < 0, when k is longer than q) and beyond the last are zero-filled
       const int lo = rbq < 0 ? 64 : -qi0, hi = sq.q_len - qi0;
@@ -405,10 +413,15 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     constexpr bool kDp = decltype(role_tag)::value;
     int issued = 0, iq = 0, ido = 0;  // next block to request and its ring positions
     bool exact = true;                // every wave has issued exactly LPT load instructions per outstanding block
-    for (int i = 0; i < S::kAhead && issued < nblk; ++i, ++issued) {
-      exact = issue(issued, iq, ido) && exact;
-      iq = iq + 1 == S::kQStages ? 0 : iq + 1;
-      ido = ido + 1 == S::kDoStages ? 0 : ido + 1;
+    static_assert(S::kAhead == 2, "the first two table entries are read together");
+    if (nblk > 0) {
+      int r0, r1;
+      scalar_load2(rows, rows + (nblk > 1 ? 1 : 0), r0, r1);  // one round trip for both
+      for (int i = 0; i < S::kAhead && issued < nblk; ++i, ++issued) {
+        exact = issue(i == 0 ? r0 : r1, iq, ido) && exact;
+        iq = iq + 1 == S::kQStages ? 0 : iq + 1;
+        ido = ido + 1 == S::kDoStages ? 0 : ido + 1;
+      }
     }
     floatx16 dp_prev;
     int cq = 0, cdo = 0, pq = 0;  // ring positions of block t (Q, dO) and of block t - 1 (Q)
@@ -416,7 +429,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       wait_tiles_ahead<LPT>(exact ? issued - t - 1 : 0);
       __syncthreads();  // block t is visible, so is P of block t - 1; the stages of block t - 2 are free
       if (issued < nblk) {
-        exact = issue(issued, iq, ido) && exact;
+        exact = issue(scalar_load(rows + issued), iq, ido) && exact;
         iq = iq + 1 == S::kQStages ? 0 : iq + 1;
         ido = ido + 1 == S::kDoStages ? 0 : ido + 1;
         ++issued;

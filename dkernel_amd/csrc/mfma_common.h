@@ -173,6 +173,13 @@ __device__ __forceinline__ int scalar_load(const int32_t *p) {
   asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(v) : "s"(uniform_address(p)) : "memory");
   return v;
 }
+// Two table reads in flight together: one round trip instead of two.
+__device__ __forceinline__ void scalar_load2(const int32_t *p0, const int32_t *p1, int &v0, int &v1) {
+  asm volatile("s_load_dword %0, %2, 0x0\n\ts_load_dword %1, %3, 0x0\n\ts_waitcnt lgkmcnt(0)"
+               : "=&s"(v0), "=&s"(v1)
+               : "s"(uniform_address(p0)), "s"(uniform_address(p1))
+               : "memory");
+}
 __device__ __forceinline__ void lds_dma16(const char *gbase, uint32_t voff, uint32_t lds_base) {
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                :

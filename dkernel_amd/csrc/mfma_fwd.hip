@@ -77,8 +77,7 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
   const int lh = lut_head(p.csr, blockIdx.x * G, p.Hq, p.Hkv);
   int e0 = 0, e1 = 0;
   if (rb < p.csr.num_rows) {  // table reads go through the scalar unit (no vector-memory wait)
-    e0 = scalar_load(p.csr.ptr + lh * p.csr.ptr_sh + rb);
-    e1 = scalar_load(p.csr.ptr + lh * p.csr.ptr_sh + rb + 1);
+    scalar_load2(p.csr.ptr + lh * p.csr.ptr_sh + rb, p.csr.ptr + lh * p.csr.ptr_sh + rb + 1, e0, e1);
   }
   const int32_t *cols = p.csr.idx + lh * p.csr.idx_sh;
   const T *kbase = (const T *)p.k.ptr + sq.b * p.k.sb + kvh * p.k.sh + (int64_t)sq.k_start * p.k.st;
@@ -299,10 +298,8 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
   }
   const int lh = lut_head(p.csr, blockIdx.x * G, p.Hq, p.Hkv);
   int e0 = 0, e1 = 0;
-  if (rb < p.csr.num_rows) {
-    e0 = p.csr.ptr[lh * p.csr.ptr_sh + rb];
-    e1 = p.csr.ptr[lh * p.csr.ptr_sh + rb + 1];
-  }
+  if (rb < p.csr.num_rows)
+    scalar_load2(p.csr.ptr + lh * p.csr.ptr_sh + rb, p.csr.ptr + lh * p.csr.ptr_sh + rb + 1, e0, e1);
   const int n = e1 - e0;
   const int32_t *cols = p.csr.idx + lh * p.csr.idx_sh + e0;
   const T *kbase = (const T *)p.k.ptr + sq.b * p.k.sb + kvh * p.k.sh + (int64_t)sq.k_start * p.k.st;

@@ -76,8 +76,8 @@ def cpu_baseline(seconds_budget=20.0):
     sm = 1.0 / math.sqrt(D)
     done_blocks, heads, t_total = 0, 0, 0.0
     tril = torch.tril(torch.ones(L, L, dtype=torch.bool))
-    while t_total < seconds_budget and heads < H:
-        h = heads
+    while t_total < seconds_budget and heads < 2 * H:  # both batch elements at most
+        h = heads % H
         q, k, v = (gen((1, 1, L, D), g, torch.bfloat16) for _ in range(3))
         mask = torch.from_numpy(bm[h]).bool().repeat_interleave(BS, 0).repeat_interleave(BS, 1) & tril
         t0 = time.perf_counter()

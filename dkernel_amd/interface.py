@@ -16,7 +16,10 @@ from torch import Tensor
 
 from .ops import _sparse_attention
 from .utils import (dense_to_ccol_row, get_sparse_attn_mask, is_kv_cache_efficient,
-                    merge_split_fwd_kernel_blocks, multiple_of, verify_sparse_pattern, zero_stride)
+                    merge_split_fwd_kernel_blocks, multiple_of, split_tile_tables, verify_sparse_pattern,
+                    zero_stride)
+
+_KERNEL_TILE = 64  # q and k tile of the matrix-core kernels
 
 
 def _identical_head_run(pattern: Tensor) -> int:
@@ -74,6 +77,9 @@ class SparseAttention(torch.nn.Module):
         _check_block_size(block_m, "block_m")
         _check_block_size(block_n, "block_n")
 
+        # Patterns with blocks larger than the 64 x 64 tile of the matrix-core kernels run on
+        # tables split to that tile, unless the caller fixes the tile sizes.
+        split_for_kernels = block_m is None and block_n is None and block_size > _KERNEL_TILE
         if block_m is None:
             block_m = max(block_size, 64) if causal else block_size
         if block_n is None:
@@ -128,6 +134,23 @@ class SparseAttention(torch.nn.Module):
         self.register_buffer("layout_csc_ccol", layout_csc[0].to(torch.int32), persistent=False)
         self.register_buffer("layout_csc_row", layout_csc[1].to(torch.int32), persistent=False)
 
+        # The layout_* buffers keep the reference's shapes; the kernels read these when present.
+        self.kernel_tile = None
+        if split_for_kernels:
+            tile_csr, tile_csc = split_tile_tables(block_size, sparse_pattern, _KERNEL_TILE, causal=causal)
+            tile_csr, tile_csc = list(tile_csr), list(tile_csc)
+            if tile_csr[0].size(0) == 1:
+                tile_csr = [zero_stride(x) for x in tile_csr]
+                tile_csc = [zero_stride(x) for x in tile_csc]
+            crow = tile_csr[0]
+            self.lut_max_row = int((crow[:, 1:] - crow[:, :-1]).max()) if crow.size(1) > 1 else 0
+            self.kwargs['lut_max_row'] = self.lut_max_row
+            self.kernel_tile = _KERNEL_TILE
+            self.register_buffer("kernel_csr_crow", tile_csr[0].to(torch.int32), persistent=False)
+            self.register_buffer("kernel_csr_col", tile_csr[1].to(torch.int32), persistent=False)
+            self.register_buffer("kernel_csc_ccol", tile_csc[0].to(torch.int32), persistent=False)
+            self.register_buffer("kernel_csc_row", tile_csc[1].to(torch.int32), persistent=False)
+
     def forward(self,
                 q: Tensor,
                 k: Optional[Tensor] = None,
@@ -159,10 +182,14 @@ class SparseAttention(torch.nn.Module):
         kwargs = copy.copy(self.kwargs)
         kwargs["return_lse"] = return_lse
         kwargs['split_qkv'] = split_qkv
+        if self.kernel_tile is not None:
+            layout_csr = (self.kernel_csr_crow, self.kernel_csr_col, self.kernel_tile, self.kernel_tile)
+            layout_csc = (self.kernel_csc_ccol, self.kernel_csc_row, self.kernel_tile, self.kernel_tile)
+        else:
+            layout_csr = (self.layout_csr_crow, self.layout_csr_col, self.block_m, self.block_n)
+            layout_csc = (self.layout_csc_ccol, self.layout_csc_row, self.block_m2, self.block_n2)
         output, lse = _sparse_attention.apply(
-            q, k, v, sm_scale,
-            (self.layout_csr_crow, self.layout_csr_col, self.block_m, self.block_n),
-            (self.layout_csc_ccol, self.layout_csc_row, self.block_m2, self.block_n2),
+            q, k, v, sm_scale, layout_csr, layout_csc,
             self.seq_dim, inf_kwargs, kwargs)
         if return_lse:
             return output, lse

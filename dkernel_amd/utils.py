@@ -196,19 +196,14 @@ def is_causal(sparse_pattern: Tensor) -> bool:
     return not upper.any()
 
 
-def merge_split_fwd_kernel_blocks(block_size: int, sparse_pattern: Tensor, block_m: int, block_n: int,
-                                  causal: bool = True) -> Tuple[Tensor, Tensor]:
-    """Look-up table at kernel-tile granularity (reference:
-    dkernel/utils.py:262-310).  `causal=False` keeps the sub-blocks above the
-    token diagonal, which the reference would drop even for bidirectional
-    patterns."""
-    if block_size == block_m and block_size == block_n:
-        return dense_to_crow_col(sparse_pattern)
+def _tile_pattern(block_size: int, sparse_pattern: Tensor, block_m: int, block_n: int,
+                  causal: bool) -> Tuple[Tensor, bool]:
+    """Block pattern re-expressed in block_m x block_n kernel tiles (int32, on
+    the CPU) and whether rows were merged (entries then hold micro_M)."""
     assert (block_m % block_size == 0) or (block_size % block_n == 0), \
         "block_m must be mutliple or a factor of sparse block size for merging on Q blocks"
     assert block_size % block_n == 0, \
         "block_n must be a factor of sparse block size for splitting on K blocks"
-    device = sparse_pattern.device
     p = (sparse_pattern != 0).to("cpu", torch.uint8).contiguous()
     H, M, N = p.shape
     lib = _lib.lib()
@@ -217,7 +212,33 @@ def merge_split_fwd_kernel_blocks(block_size: int, sparse_pattern: Tensor, block
                                          C.byref(om), C.byref(on), C.byref(merged)))
     out = torch.empty((H, om.value, on.value), dtype=torch.int32)
     _lib.check(lib.dk_tile_pattern(_ptr(p), H, M, N, block_size, block_m, block_n, int(bool(causal)), _ptr(out)))
-    return dense_to_crow_col(out.to(device), include_values=bool(merged.value))
+    return out, bool(merged.value)
+
+
+def merge_split_fwd_kernel_blocks(block_size: int, sparse_pattern: Tensor, block_m: int, block_n: int,
+                                  causal: bool = True) -> Tuple[Tensor, Tensor]:
+    """Look-up table at kernel-tile granularity (reference:
+    dkernel/utils.py:262-310).  `causal=False` keeps the sub-blocks above the
+    token diagonal, which the reference would drop even for bidirectional
+    patterns."""
+    if block_size == block_m and block_size == block_n:
+        return dense_to_crow_col(sparse_pattern)
+    out, merged = _tile_pattern(block_size, sparse_pattern, block_m, block_n, causal)
+    return dense_to_crow_col(out.to(sparse_pattern.device), include_values=merged)
+
+
+def split_tile_tables(block_size: int, sparse_pattern: Tensor, tile: int,
+                      causal: bool = True) -> Tuple[Tuple[Tensor, Tensor], Tuple[Tensor, Tensor]]:
+    """CSR and CSC tables of a pattern whose blocks are split into tile x tile
+    kernel tiles (tile divides block_size).  With `causal`, tiles that lie
+    entirely above the token diagonal are dropped, as in
+    `merge_split_fwd_kernel_blocks`.  The reference has no counterpart: its
+    dK/dV pass always walks columns of block_size (dkernel/interface.py:134)."""
+    assert block_size % tile == 0 and block_size > tile
+    out, merged = _tile_pattern(block_size, sparse_pattern, tile, tile, causal)
+    assert not merged
+    out = out.to(sparse_pattern.device)
+    return dense_to_crow_col(out), dense_to_ccol_row(out)
 
 
 def zero_stride(x: Tensor, dim=0) -> Tensor:

@@ -137,6 +137,20 @@ def test_kernel_tile_sizes(impl, bs, bm, bn):
     run_fwd_bwd(1, 2, 2, 1024, 128, torch.bfloat16, bs, 1, 4, block_m=bm, block_n=bn)
 
 
+@pytest.mark.parametrize("bs,D,dtype", [(128, 128, torch.bfloat16), (256, 128, torch.bfloat16),
+                                        (128, 64, torch.float16)])
+def test_large_blocks_run_on_split_tiles(impl, bs, D, dtype):
+    """Pattern blocks of 128 / 256 are split into the 64 x 64 tiles of the
+    matrix-core kernels (forward CSR and backward CSC); results must equal the
+    dense oracle of the unsplit pattern."""
+    mod = _module(8, 1024, bs, 2, 4, num_kv_heads=2)
+    assert mod.kernel_tile == 64 and mod.block_m == bs and mod.block_n == bs
+    assert mod.kernel_csr_crow.shape[-1] == 1024 // 64 + 1
+    run_fwd_bwd(2, 8, 2, 1024, D, dtype, bs, 2, 4)
+    run_fwd_bwd(1, 4, 4, 1000, D, dtype, bs, 1, 3, num_dense_heads=1)
+    run_fwd_bwd(1, 2, 2, 1024, D, dtype, bs, 2, 4, causal=False)
+
+
 def test_grad_through_lse(impl):
     run_fwd_bwd(1, 4, 4, 512, 64, torch.float32, 64, 2, 4, with_dlse=True)
     run_fwd_bwd(1, 4, 2, 512, 128, torch.bfloat16, 64, 2, 4, with_dlse=True)
@@ -208,7 +222,8 @@ def test_right_padded_prefill(impl):
         assert (out[i, :, l:] == 0).all()
 
 
-@pytest.mark.parametrize("bs,block_m,left", [(64, None, True), (32, None, True), (16, 128, False), (64, None, False)])
+@pytest.mark.parametrize("bs,block_m,left", [(64, None, True), (32, None, True), (16, 128, False), (64, None, False),
+                                             (128, None, True)])
 def test_decode(impl, bs, block_m, left):
     """One new token per sequence over left-padded / right-padded / unpadded KV, GQA."""
     B, Hq, Hkv, Lmax, D = 4, 8, 2, 2048, 128

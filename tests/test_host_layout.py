@@ -151,6 +151,29 @@ def test_module_construction_matches_reference_surface():
         LocalStrideSparseAttention(8, 1024, 64, 0, 8)
 
 
+@pytest.mark.parametrize("bs,causal", [(128, True), (256, True), (128, False)])
+def test_large_blocks_get_split_kernel_tables(bs, causal):
+    """Blocks larger than the 64 x 64 kernel tile: the layout_* buffers keep the
+    reference's shapes, the kernel tables are the pattern expanded to 64 x 64
+    tiles (tiles above the token diagonal dropped when causal), as CSR and CSC."""
+    L, H = 2048, 4
+    m = LocalStrideSparseAttention(H, L, bs, 2, 4, causal=causal)
+    assert m.kernel_tile == 64 and (m.block_m, m.block_n, m.block_m2, m.block_n2) == (bs, bs, bs, bs)
+    pattern = np.asarray(OL.block_mask(H, L, bs, 2, 4, causal=causal)) != 0
+    assert m.layout_csr_crow.shape == (pattern.shape[0], L // bs + 1)
+    f = bs // 64
+    want = np.kron(pattern, np.ones((f, f), dtype=bool))
+    if causal:
+        want = np.tril(want)
+    got_csr = U.crow_col_to_dense(m.kernel_csr_crow, m.kernel_csr_col, torch.uint8).numpy() != 0
+    got_csc = U.ccol_row_to_dense(m.kernel_csc_ccol, m.kernel_csc_row, torch.uint8).numpy() != 0
+    assert np.array_equal(got_csr, want) and np.array_equal(got_csc, want)
+    assert m.lut_max_row == int(want.sum(-1).max())
+    # explicit tile sizes are honoured as given
+    assert LocalStrideSparseAttention(H, L, bs, 2, 4, causal=causal, block_m=bs, block_n=64).kernel_tile is None
+    assert LocalStrideSparseAttention(H, L, 64, 2, 4, causal=causal).kernel_tile is None
+
+
 def test_cpu_tensors_are_refused_loudly():
     m = LocalStrideSparseAttention(2, 128, 64, 1, 2)
     x = torch.zeros(1, 128, 2, 64)

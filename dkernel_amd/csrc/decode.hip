@@ -47,7 +47,7 @@ struct DecSmem {  // per wave: one 32-key half block of K and of V, plus q of th
 };
 
 // workspace layout: [batch][Hq][max_units][D + 2] floats (O[D] unnormalised, max, sum)
-template <typename T, int D>
+template <typename T, int D, bool PAD>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void decode_partial_kernel(const FwdParams p, float *ws, int unit_blocks,
                                                             int max_units) {
   using M = Mma<T>;
@@ -82,7 +82,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
   uint4 kreg[HCH], vreg[HCH];
   auto prefetch = [&](int hb, int col) {
     const int key0 = col * 64 + (hb & 1) * 32;
-    if (col >= 0 && key0 + 32 <= sq.k_len) {  // whole half inside the sequence: no per-row guards
+    if (!PAD && col >= 0 && key0 + 32 <= sq.k_len) {  // whole half inside the sequence: no guards
 #pragma unroll
       for (int c = 0; c < HCH; ++c) {
         const int idx = lane + c * 64;
@@ -90,13 +90,13 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
         kreg[c] = *reinterpret_cast<const uint4 *>(kbase + (int64_t)(key0 + r) * p.k.st + ch * 8);
         vreg[c] = *reinterpret_cast<const uint4 *>(vbase + (int64_t)(key0 + r) * p.v.st + ch * 8);
       }
-    } else {
+    } else {  // rows beyond the sequence and (PAD) head dims beyond p.D read as zeros
 #pragma unroll
       for (int c = 0; c < HCH; ++c) {
         const int idx = lane + c * 64;
         const int r = idx / CPR, ch = idx % CPR;
         kreg[c] = vreg[c] = make_uint4(0, 0, 0, 0);
-        if (col >= 0 && key0 + r < sq.k_len) {
+        if (col >= 0 && key0 + r < sq.k_len && (!PAD || ch * 8 < p.D)) {
           kreg[c] = *reinterpret_cast<const uint4 *>(kbase + (int64_t)(key0 + r) * p.k.st + ch * 8);
           vreg[c] = *reinterpret_cast<const uint4 *>(vbase + (int64_t)(key0 + r) * p.v.st + ch * 8);
         }
@@ -114,7 +114,9 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
     const int hh = lane / CPR, ch = lane % CPR;  // 64 lanes cover 64 / CPR heads per pass
     for (int h = hh; h < ratio; h += 64 / CPR) {
       const T *qp = (const T *)p.q.ptr + sq.b * p.q.sb + (int64_t)(h0 + h) * p.q.sh + (int64_t)sq.q_start * p.q.st;
-      *reinterpret_cast<uint4 *>(qs_ + h * D * 2 + ch * 16) = *reinterpret_cast<const uint4 *>(qp + ch * 8);
+      uint4 w = make_uint4(0, 0, 0, 0);
+      if (!PAD || ch * 8 < p.D) w = *reinterpret_cast<const uint4 *>(qp + ch * 8);
+      *reinterpret_cast<uint4 *>(qs_ + h * D * 2 + ch * 16) = w;
     }
   }
   const int q_read = (m < ratio ? m : ratio - 1) * D * 2 + g * 16;
@@ -230,7 +232,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
 // dims {2l, 2l+1} (D = 128) or dim l (D = 64).  All loads of a row are issued
 // before the first use (units are few, a dependent load chain per unit would
 // make this small kernel latency-bound).
-template <typename T, int D>
+template <typename T, int D, bool PAD>
 __global__ __launch_bounds__(64) void decode_combine_kernel(const FwdParams p, const float *ws, int unit_blocks,
                                                             int max_units) {
   constexpr int PER = D / 64;  // dims per lane
@@ -280,7 +282,8 @@ __global__ __launch_bounds__(64) void decode_combine_kernel(const FwdParams p, c
   const float inv = l > 0.f ? 1.f / l : 0.f;
   T *op = (T *)p.o.ptr + sq.b * p.o.sb + h * p.o.sh + (int64_t)sq.q_start * p.o.st;
 #pragma unroll
-  for (int i = 0; i < PER; ++i) op[lane * PER + i] = from_float<T>(o[i] * inv);
+  for (int i = 0; i < PER; ++i)
+    if (!PAD || lane * PER + i < p.D) op[lane * PER + i] = from_float<T>(o[i] * inv);
   if (p.lse.ptr && lane == 0)
     p.lse.ptr[sq.b * p.lse.sb + h * p.lse.sh + (int64_t)sq.q_start * p.lse.st] =
         l > 0.f ? (mmax + log2f(l)) * kLn2 : -INFINITY;
@@ -297,36 +300,42 @@ bool decode_supported(const FwdParams &p, int dtype) {
   const int ratio = p.Hq / p.Hkv;
   const bool shared_row = p.csr.num_heads == 1 || (p.csr.num_heads == p.Hkv && p.Hkv != p.Hq) || ratio == 1 ||
                           (p.csr.num_heads == p.Hq && p.csr.group % ratio == 0);
-  return (dtype == DK_BF16 || dtype == DK_F16) && (p.D == 128 || p.D == 64) && p.csr.block_rows == 64 &&
+  return (dtype == DK_BF16 || dtype == DK_F16) && mfma_head_dim_ok(p.D) && p.csr.block_rows == 64 &&
          p.csr.block_cols == 64 && p.csr.entry_width == 1 && p.vec_ok && !p.seqs.packed &&
          p.seqs.max_q_len == 1 && ratio <= 32 && shared_row && p.causal;
 }
 
 size_t decode_workspace_bytes(const FwdParams &p) {
-  return (size_t)p.seqs.batch * p.Hq * decode_max_units(p) * (p.D + 2) * sizeof(float);
+  return (size_t)p.seqs.batch * p.Hq * decode_max_units(p) * (mfma_tile_width(p.D) + 2) * sizeof(float);
 }
 
-template <typename T, int D>
+template <typename T, int D, bool PAD>
 static int launch_decode_td(const FwdParams &p, float *ws, hipStream_t stream) {
   const int smem = DecSmem<D>::wave_bytes(p.Hq / p.Hkv);
   const int unit_blocks = decode_unit_blocks(), max_units = decode_max_units(p);
   DK_REQUIRE(max_units <= 65535, "too many decode units");
-  hipLaunchKernelGGL((decode_partial_kernel<T, D>), dim3(max_units, p.Hkv, p.seqs.batch), dim3(64), smem, stream,
+  hipLaunchKernelGGL((decode_partial_kernel<T, D, PAD>), dim3(max_units, p.Hkv, p.seqs.batch), dim3(64), smem, stream,
                      p, ws, unit_blocks, max_units);
   DK_HIP_CHECK(hipGetLastError());
-  hipLaunchKernelGGL((decode_combine_kernel<T, D>), dim3(p.Hq, p.seqs.batch), dim3(64), 0, stream, p, ws,
+  hipLaunchKernelGGL((decode_combine_kernel<T, D, PAD>), dim3(p.Hq, p.seqs.batch), dim3(64), 0, stream, p, ws,
                      unit_blocks, max_units);
   DK_HIP_CHECK(hipGetLastError());
   return DK_OK;
+}
+
+// head dims below the tile width (64 or 128) run the zero-padded instantiation
+template <typename T>
+static int launch_decode_t(const FwdParams &p, float *ws, hipStream_t stream) {
+  if (p.D == 128) return launch_decode_td<T, 128, false>(p, ws, stream);
+  if (p.D == 64) return launch_decode_td<T, 64, false>(p, ws, stream);
+  return p.D > 64 ? launch_decode_td<T, 128, true>(p, ws, stream) : launch_decode_td<T, 64, true>(p, ws, stream);
 }
 
 int launch_decode(const FwdParams &p, int dtype, void *workspace, size_t workspace_bytes, hipStream_t stream) {
   DK_REQUIRE(workspace && workspace_bytes >= decode_workspace_bytes(p), "decode workspace too small");
   DK_REQUIRE(((uintptr_t)workspace % 16) == 0, "decode workspace must be 16-byte aligned");
   float *ws = (float *)workspace;
-  if (dtype == DK_BF16)
-    return p.D == 128 ? launch_decode_td<bf16_t, 128>(p, ws, stream) : launch_decode_td<bf16_t, 64>(p, ws, stream);
-  return p.D == 128 ? launch_decode_td<f16_t, 128>(p, ws, stream) : launch_decode_td<f16_t, 64>(p, ws, stream);
+  return dtype == DK_BF16 ? launch_decode_t<bf16_t>(p, ws, stream) : launch_decode_t<f16_t>(p, ws, stream);
 }
 
 }  // namespace dk

@@ -43,7 +43,7 @@ struct BoolConst {
 // ---------------------------------------------------------------------------
 // dQ pass
 // ---------------------------------------------------------------------------
-template <typename T, int D>
+template <typename T, int D, bool PAD>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void mfma_dq_kernel(const BwdParams p,
                                                                                                    int tiles_y) {
   using M = Mma<T>;
@@ -68,6 +68,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int pos = row0 + m;
   const int qi = pos - sq.past;
   const bool row_ok = qi >= 0 && qi < sq.q_len;
+  if constexpr (PAD) {  // the slots of the head dims beyond p.D stay zero for the whole kernel
+    zero_tiles<NT>(smem, 2 * STAGE, tid);
+    __syncthreads();
+  }
 
   // Row data of this lane (Q, dO, O fragments, lse, dLSE) is requested before anything else, so
   // that its round trip overlaps with the table reads and the first tile request; it is used
@@ -81,7 +85,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       qraw[ks] = doraw[ks] = oraw[ks] = make_uint4(0, 0, 0, 0);
-      if (row_ok) {
+      if (row_ok && (!PAD || ks * 16 + g * 8 < p.D)) {
         qraw[ks] = *reinterpret_cast<const uint4 *>(qp + ks * 16 + g * 8);
         doraw[ks] = *reinterpret_cast<const uint4 *>(dop + ks * 16 + g * 8);
         oraw[ks] = *reinterpret_cast<const uint4 *>(op + ks * 16 + g * 8);
@@ -104,9 +108,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const T *kbase = (const T *)p.k.ptr + sq.b * p.k.sb + kvh * p.k.sh;
   const T *vbase = (const T *)p.v.ptr + sq.b * p.v.sb + kvh * p.v.sh;
 
-  TileLoader<D, NT> kload, vload;
-  kload.init(tid, p.k.st);
-  vload.init(tid, p.v.st);
+  TileLoader<D, NT, PAD> kload, vload;
+  kload.init(tid, p.k.st, p.D);
+  vload.init(tid, p.v.st, p.D);
   auto issue = [&](int col, int stage) {  // asynchronous copy of K/V block `col` into `stage`
     const int key0 = col * 64;
     const int valid = col < 0 ? 0 : sq.k_len - key0;
@@ -253,7 +257,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         const int r = r4 * 4 + i;
         o4[i] = from_float<T>((acc[dt][r] + red[((rh * DT + dt) * 16 + r) * 64 + lane]) * p.sm_scale);
       }
-      *reinterpret_cast<uint2 *>(dqp + dt * 32 + r4 * 8 + g * 4) = *reinterpret_cast<const uint2 *>(o4);
+      if (!PAD || dt * 32 + r4 * 8 + g * 4 < p.D)
+        *reinterpret_cast<uint2 *>(dqp + dt * 32 + r4 * 8 + g * 4) = *reinterpret_cast<const uint2 *>(o4);
     }
 }
 
@@ -285,7 +290,7 @@ struct DkdvSmem {
   static constexpr int kBytes = kLoop > kRed ? kLoop : kRed;
 };
 
-template <typename T, int D>
+template <typename T, int D, bool PAD>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void mfma_dkdv_kernel(const BwdParams p) {
   using M = Mma<T>;
   using vec8 = typename M::vec8;
@@ -317,7 +322,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       uint4 a = make_uint4(0, 0, 0, 0);
-      if (key_ok) a = *reinterpret_cast<const uint4 *>(src + ks * 16 + g * 8);
+      if (key_ok && (!PAD || ks * 16 + g * 8 < p.D)) a = *reinterpret_cast<const uint4 *>(src + ks * 16 + g * 8);
       kvf[ks] = as_vec8<vec8>(a);
     }
   }
@@ -327,9 +332,13 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[dt][r] = 0.f;
 
-  TileLoader<D, NT> qload, doload;
-  qload.init(tid, p.q.st);
-  doload.init(tid, p.dout.st);
+  TileLoader<D, NT, PAD> qload, doload;
+  qload.init(tid, p.q.st, p.D);
+  doload.init(tid, p.dout.st, p.D);
+  if constexpr (PAD) {  // the slots of the head dims beyond p.D stay zero in every Q / dO stage
+    zero_tiles<NT>(smem, S::kVec, tid);
+    __syncthreads();
+  }
   int rd[KS], tr[DT][2];
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) rd[ks] = TL::off(mh * 32 + n, 2 * ks + g);
@@ -552,37 +561,46 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         const int r = r4 * 4 + i;
         o4[i] = from_float<T>((acc[dt][r] + red[(dt * 16 + r) * 64 + lane]) * out_scale);
       }
-      *reinterpret_cast<uint2 *>(outp + dt * 32 + r4 * 8 + g * 4) = *reinterpret_cast<const uint2 *>(o4);
+      if (!PAD || dt * 32 + r4 * 8 + g * 4 < p.D)
+        *reinterpret_cast<uint2 *>(outp + dt * 32 + r4 * 8 + g * 4) = *reinterpret_cast<const uint2 *>(o4);
     }
 }
 
 // Explicit instantiations: with only the implicit ones the fp16 host stubs of
 // these kernels are not emitted by this compiler version.
-template __global__ void mfma_dq_kernel<bf16_t, 128>(const BwdParams, int);
-template __global__ void mfma_dq_kernel<bf16_t, 64>(const BwdParams, int);
-template __global__ void mfma_dq_kernel<f16_t, 128>(const BwdParams, int);
-template __global__ void mfma_dq_kernel<f16_t, 64>(const BwdParams, int);
-template __global__ void mfma_dkdv_kernel<bf16_t, 128>(const BwdParams);
-template __global__ void mfma_dkdv_kernel<bf16_t, 64>(const BwdParams);
-template __global__ void mfma_dkdv_kernel<f16_t, 128>(const BwdParams);
-template __global__ void mfma_dkdv_kernel<f16_t, 64>(const BwdParams);
+template __global__ void mfma_dq_kernel<bf16_t, 128, false>(const BwdParams, int);
+template __global__ void mfma_dq_kernel<bf16_t, 128, true>(const BwdParams, int);
+template __global__ void mfma_dq_kernel<bf16_t, 64, false>(const BwdParams, int);
+template __global__ void mfma_dq_kernel<bf16_t, 64, true>(const BwdParams, int);
+template __global__ void mfma_dq_kernel<f16_t, 128, false>(const BwdParams, int);
+template __global__ void mfma_dq_kernel<f16_t, 128, true>(const BwdParams, int);
+template __global__ void mfma_dq_kernel<f16_t, 64, false>(const BwdParams, int);
+template __global__ void mfma_dq_kernel<f16_t, 64, true>(const BwdParams, int);
+template __global__ void mfma_dkdv_kernel<bf16_t, 128, false>(const BwdParams);
+template __global__ void mfma_dkdv_kernel<bf16_t, 128, true>(const BwdParams);
+template __global__ void mfma_dkdv_kernel<bf16_t, 64, false>(const BwdParams);
+template __global__ void mfma_dkdv_kernel<bf16_t, 64, true>(const BwdParams);
+template __global__ void mfma_dkdv_kernel<f16_t, 128, false>(const BwdParams);
+template __global__ void mfma_dkdv_kernel<f16_t, 128, true>(const BwdParams);
+template __global__ void mfma_dkdv_kernel<f16_t, 64, false>(const BwdParams);
+template __global__ void mfma_dkdv_kernel<f16_t, 64, true>(const BwdParams);
 
 bool mfma_bwd_supported(const BwdParams &p, int dtype) {
-  return (dtype == DK_BF16 || dtype == DK_F16) && (p.D == 128 || p.D == 64) && p.csr.block_rows == 64 &&
+  return (dtype == DK_BF16 || dtype == DK_F16) && mfma_head_dim_ok(p.D) && p.csr.block_rows == 64 &&
          p.csr.block_cols == 64 && p.csr.entry_width == 1 && p.csc.block_rows == 64 && p.csc.block_cols == 64 &&
          p.vec_ok;
 }
 
-template <typename T, int D>
+template <typename T, int D, bool PAD>
 static int launch_bwd_td(const BwdParams &p, hipStream_t stream) {
   const SeqView &s = p.seqs;
   constexpr int smem_dq = 2 * 2 * Tile<D>::kBytes;
   constexpr int smem_dkdv = DkdvSmem<D>::kBytes;
   static bool attr_set = false;
   if (!attr_set) {
-    DK_HIP_CHECK(hipFuncSetAttribute((const void *)mfma_dq_kernel<T, D>,
+    DK_HIP_CHECK(hipFuncSetAttribute((const void *)mfma_dq_kernel<T, D, PAD>,
                                      hipFuncAttributeMaxDynamicSharedMemorySize, smem_dq));
-    DK_HIP_CHECK(hipFuncSetAttribute((const void *)mfma_dkdv_kernel<T, D>,
+    DK_HIP_CHECK(hipFuncSetAttribute((const void *)mfma_dkdv_kernel<T, D, PAD>,
                                      hipFuncAttributeMaxDynamicSharedMemorySize, smem_dkdv));
     attr_set = true;
   }
@@ -591,17 +609,23 @@ static int launch_bwd_td(const BwdParams &p, hipStream_t stream) {
   const int cblocks = cdiv(s.max_k_len, 64);
   DK_REQUIRE(tiles <= 65535 && cblocks <= 65535, "sequence too long for one launch");
   // dQ first: it also writes delta, which the dK/dV pass reads
-  hipLaunchKernelGGL((mfma_dq_kernel<T, D>), dim3(p.Hq, tiles, s.batch), dim3(256), smem_dq, stream, p, tiles);
+  hipLaunchKernelGGL((mfma_dq_kernel<T, D, PAD>), dim3(p.Hq, tiles, s.batch), dim3(256), smem_dq, stream, p, tiles);
   DK_HIP_CHECK(hipGetLastError());
-  hipLaunchKernelGGL((mfma_dkdv_kernel<T, D>), dim3(p.Hkv, cblocks, s.batch), dim3(512), smem_dkdv, stream, p);
+  hipLaunchKernelGGL((mfma_dkdv_kernel<T, D, PAD>), dim3(p.Hkv, cblocks, s.batch), dim3(512), smem_dkdv, stream, p);
   DK_HIP_CHECK(hipGetLastError());
   return DK_OK;
 }
 
+// head dims below the tile width (64 or 128) run the zero-padded instantiation
+template <typename T>
+static int launch_bwd_t(const BwdParams &p, hipStream_t stream) {
+  if (p.D == 128) return launch_bwd_td<T, 128, false>(p, stream);
+  if (p.D == 64) return launch_bwd_td<T, 64, false>(p, stream);
+  return p.D > 64 ? launch_bwd_td<T, 128, true>(p, stream) : launch_bwd_td<T, 64, true>(p, stream);
+}
+
 int launch_mfma_bwd(const BwdParams &p, int dtype, hipStream_t stream) {
-  if (dtype == DK_BF16)
-    return p.D == 128 ? launch_bwd_td<bf16_t, 128>(p, stream) : launch_bwd_td<bf16_t, 64>(p, stream);
-  return p.D == 128 ? launch_bwd_td<f16_t, 128>(p, stream) : launch_bwd_td<f16_t, 64>(p, stream);
+  return dtype == DK_BF16 ? launch_bwd_t<bf16_t>(p, stream) : launch_bwd_t<f16_t>(p, stream);
 }
 
 }  // namespace dk

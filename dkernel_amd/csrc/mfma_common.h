@@ -20,6 +20,12 @@
 
 namespace dk {
 
+// Head dims the MFMA kernels take: multiples of 8 up to 128.  They run at a
+// tile width of 64 or 128; narrower rows are zero-padded on chip.
+__host__ __device__ inline bool mfma_head_dim_ok(int d) { return d >= 8 && d <= 128 && d % 8 == 0; }
+__host__ __device__ inline int mfma_tile_width(int d) { return d <= 64 ? 64 : 128; }
+
+
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -200,25 +206,36 @@ __device__ __forceinline__ void lds_dma4(const char *gbase, uint32_t voff, uint3
 // TileLoader::init computes the per-thread global byte offsets once.  Rows
 // outside [lo, hi) are zero-filled with ordinary LDS stores.  The caller
 // waits (wait_tile_loads) and synchronises before reading the tile.
-template <int D, int NT>
+//
+// PAD: the rows in memory hold fewer than D elements (a head_dim that is a
+// multiple of 8 below the tile width).  Lanes whose chunk lies beyond the real
+// width copy nothing; their LDS slots are never written by any copy, so a
+// tile area that was zeroed once (zero_tiles) keeps zeros there for good.
+// Every row has chunks inside the real width, so every wave still issues
+// exactly kChunks load instructions per tile.
+template <int D, int NT, bool PAD = false>
 struct TileLoader {
   static constexpr int kCPR = D / 8;
   static constexpr int kChunks = 64 * kCPR / NT;
   uint32_t goff[kChunks];  // global byte offset of this thread's chunk c inside the 64-row block
   int row0;                // first row this thread's wave covers with chunk 0 (wave-uniform)
   int lane_row, lane_byte;
+  uint32_t inside;         // PAD: bit c set when this thread's chunk c lies inside the real width
 
-  __device__ __forceinline__ void init(int tid, int64_t row_stride_elems) {
+  __device__ __forceinline__ void init(int tid, int64_t row_stride_elems, int real_d = D) {
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     row0 = wave * (64 / kCPR);
     lane_row = lane / kCPR;
     lane_byte = lane * 16;
+    inside = 0;
 #pragma unroll
     for (int c = 0; c < kChunks; ++c) {
       const int r = row0 + c * (NT / kCPR) + lane_row;
       const int pos = lane % kCPR;
-      goff[c] = (uint32_t)(r * row_stride_elems) * 2u + (uint32_t)((pos ^ Tile<D>::swz(r)) << 4);
+      const int chunk = pos ^ Tile<D>::swz(r);
+      goff[c] = (uint32_t)(r * row_stride_elems) * 2u + (uint32_t)(chunk << 4);
+      if (chunk * 8 < real_d) inside |= 1u << c;
     }
   }
   // rows [lo, hi) of the block are copied, the others zero-filled.  Returns true when the
@@ -228,22 +245,30 @@ struct TileLoader {
     const uint32_t base = lds_address(tile) + row0 * Tile<D>::kRowBytes;
     if (lo <= 0 && hi >= 64) {
 #pragma unroll
-      for (int c = 0; c < kChunks; ++c) lds_dma16(gblk, goff[c], base + c * (NT / kCPR) * Tile<D>::kRowBytes);
+      for (int c = 0; c < kChunks; ++c)
+        if (!PAD || ((inside >> c) & 1)) lds_dma16(gblk, goff[c], base + c * (NT / kCPR) * Tile<D>::kRowBytes);
       return true;
     } else {
 #pragma unroll
       for (int c = 0; c < kChunks; ++c) {
         char *wbase = tile + (row0 + c * (NT / kCPR)) * Tile<D>::kRowBytes;
         const int r = row0 + c * (NT / kCPR) + lane_row;
-        if (r >= lo && r < hi)
-          lds_dma16(gblk, goff[c], base + c * (NT / kCPR) * Tile<D>::kRowBytes);
-        else
+        if (r >= lo && r < hi) {
+          if (!PAD || ((inside >> c) & 1)) lds_dma16(gblk, goff[c], base + c * (NT / kCPR) * Tile<D>::kRowBytes);
+        } else {
           *reinterpret_cast<uint4 *>(wbase + lane_byte) = make_uint4(0, 0, 0, 0);
+        }
       }
       return false;
     }
   }
 };
+
+// Zero `bytes` (a multiple of 16) of LDS with NT threads; the caller synchronises afterwards.
+template <int NT>
+__device__ __forceinline__ void zero_tiles(char *lds, int bytes, int tid) {
+  for (int off = tid * 16; off < bytes; off += NT * 16) *reinterpret_cast<uint4 *>(lds + off) = make_uint4(0, 0, 0, 0);
+}
 
 // All asynchronous tile loads (and any other vector memory loads) of this wave have landed.
 __device__ __forceinline__ void wait_tile_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }

@@ -37,7 +37,7 @@ struct FwdSmem {  // one stage = K tile + V tile, swizzled row-major (mfma_commo
   static constexpr int kStage = 2 * Tile<D>::kBytes;
 };
 
-template <typename T, int D, int G>
+template <typename T, int D, int G, bool PAD>
 __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 ? 1 : 2, 2))) void mfma_fwd_kernel(const FwdParams p, int tiles_y) {
   using M = Mma<T>;
   using vec8 = typename M::vec8;
@@ -54,6 +54,10 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
   if (!resolve_tile(p.seqs, p.causal, 64, 1, ty, blockIdx.z, sq, tile)) return;
   const int rb = sq.past / 64 + tile;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  if constexpr (PAD) {  // the slots of the head dims beyond p.D stay zero for the whole kernel
+    zero_tiles<NT>(smem, 2 * S::kStage, tid);
+    __syncthreads();
+  }
   const int h = blockIdx.x * G + (wave >> 1);
   const int kvh = __builtin_amdgcn_readfirstlane(h / (p.Hq / p.Hkv));  // integer division runs on the VALU
   const int m = lane & 31, g = lane >> 5;
@@ -69,7 +73,7 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       uint4 w = make_uint4(0, 0, 0, 0);
-      if (row_ok) w = *reinterpret_cast<const uint4 *>(qp + ks * 16 + g * 8);
+      if (row_ok && (!PAD || ks * 16 + g * 8 < p.D)) w = *reinterpret_cast<const uint4 *>(qp + ks * 16 + g * 8);
       qf[ks] = as_vec8<vec8>(w);
     }
   }
@@ -84,9 +88,9 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
   const T *vbase = (const T *)p.v.ptr + sq.b * p.v.sb + kvh * p.v.sh + (int64_t)sq.k_start * p.v.st;
 
   // ---- asynchronous HBM -> LDS copy of one K/V tile pair (no staging registers) ----
-  TileLoader<D, NT> kload, vload;
-  kload.init(tid, p.k.st);
-  vload.init(tid, p.v.st);
+  TileLoader<D, NT, PAD> kload, vload;
+  kload.init(tid, p.k.st, p.D);
+  vload.init(tid, p.v.st, p.D);
   auto issue = [&](int col, int stage) {
     const int key0 = col * 64;
     const int valid = col < 0 ? 0 : sq.k_len - key0;
@@ -244,7 +248,8 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
       T o4[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) o4[i] = from_float<T>(oacc[dt][r4 * 4 + i] * inv);
-      *reinterpret_cast<uint2 *>(op + dt * 32 + r4 * 8 + g * 4) = *reinterpret_cast<const uint2 *>(o4);
+      if (!PAD || dt * 32 + r4 * 8 + g * 4 < p.D)
+        *reinterpret_cast<uint2 *>(op + dt * 32 + r4 * 8 + g * 4) = *reinterpret_cast<const uint2 *>(o4);
     }
   if (p.lse.ptr && g == 0) {
     const float lse = l_run > 0.f ? (m_run + log2f(l_run)) * kLn2 : -INFINITY;
@@ -260,7 +265,7 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
 // stages.  Same work split, grid and results as mfma_fwd_kernel.  Used for
 // one head per workgroup (G = 1, one wave per SIMD), where it measures faster.
 // ---------------------------------------------------------------------------
-template <typename T, int D, int G>
+template <typename T, int D, int G, bool PAD>
 __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 ? 1 : 2, 2))) void mfma_fwd_pipe_kernel(
     const FwdParams p, int tiles_y) {
   using M = Mma<T>;
@@ -278,6 +283,10 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
   const int rb = sq.past / 64 + tile;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  if constexpr (PAD) {  // the slots of the head dims beyond p.D stay zero for the whole kernel
+    zero_tiles<NT>(smem, 4 * TL::kBytes, tid);
+    __syncthreads();
+  }
   const int h = blockIdx.x * G + (wave >> 1);
   const int kvh = __builtin_amdgcn_readfirstlane(h / (p.Hq / p.Hkv));  // integer division runs on the VALU
   const int m = lane & 31, g = lane >> 5;
@@ -292,7 +301,7 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       uint4 w = make_uint4(0, 0, 0, 0);
-      if (row_ok) w = *reinterpret_cast<const uint4 *>(qp + ks * 16 + g * 8);
+      if (row_ok && (!PAD || ks * 16 + g * 8 < p.D)) w = *reinterpret_cast<const uint4 *>(qp + ks * 16 + g * 8);
       qf[ks] = as_vec8<vec8>(w);
     }
   }
@@ -305,9 +314,9 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
   const T *kbase = (const T *)p.k.ptr + sq.b * p.k.sb + kvh * p.k.sh + (int64_t)sq.k_start * p.k.st;
   const T *vbase = (const T *)p.v.ptr + sq.b * p.v.sb + kvh * p.v.sh + (int64_t)sq.k_start * p.v.st;
 
-  TileLoader<D, NT> kload, vload;
-  kload.init(tid, p.k.st);
-  vload.init(tid, p.v.st);
+  TileLoader<D, NT, PAD> kload, vload;
+  kload.init(tid, p.k.st, p.D);
+  vload.init(tid, p.v.st, p.D);
   // table entries are read well before they are needed and never between a tile request and
   // its wait (a vector load there would make the wait cover the tile just requested)
   auto col_at = [&](int j) { return __builtin_amdgcn_readfirstlane(j < n ? cols[j] : 0); };
@@ -498,7 +507,8 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
       T o4[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) o4[i] = from_float<T>(oacc[dt][r4 * 4 + i] * inv);
-      *reinterpret_cast<uint2 *>(op + dt * 32 + r4 * 8 + g * 4) = *reinterpret_cast<const uint2 *>(o4);
+      if (!PAD || dt * 32 + r4 * 8 + g * 4 < p.D)
+        *reinterpret_cast<uint2 *>(op + dt * 32 + r4 * 8 + g * 4) = *reinterpret_cast<const uint2 *>(o4);
     }
   if (p.lse.ptr && g == 0) {
     const float lse = l_run > 0.f ? (m_run + log2f(l_run)) * kLn2 : -INFINITY;
@@ -508,15 +518,19 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
 
 // Explicit instantiations: with only the implicit ones the fp16 host stubs of
 // this kernel are not emitted by this compiler version.
-#define DK_INSTANTIATE_FWD(T, D)                                                  \
-  template __global__ void mfma_fwd_kernel<T, D, 1>(const FwdParams, int);       \
-  template __global__ void mfma_fwd_kernel<T, D, 2>(const FwdParams, int);       \
-  template __global__ void mfma_fwd_kernel<T, D, 4>(const FwdParams, int);       \
-  template __global__ void mfma_fwd_pipe_kernel<T, D, 1>(const FwdParams, int);
-DK_INSTANTIATE_FWD(bf16_t, 128)
-DK_INSTANTIATE_FWD(bf16_t, 64)
-DK_INSTANTIATE_FWD(f16_t, 128)
-DK_INSTANTIATE_FWD(f16_t, 64)
+#define DK_INSTANTIATE_FWD(T, D, PAD)                                                  \
+  template __global__ void mfma_fwd_kernel<T, D, 1, PAD>(const FwdParams, int);       \
+  template __global__ void mfma_fwd_kernel<T, D, 2, PAD>(const FwdParams, int);       \
+  template __global__ void mfma_fwd_kernel<T, D, 4, PAD>(const FwdParams, int);       \
+  template __global__ void mfma_fwd_pipe_kernel<T, D, 1, PAD>(const FwdParams, int);
+DK_INSTANTIATE_FWD(bf16_t, 128, false)
+DK_INSTANTIATE_FWD(bf16_t, 64, false)
+DK_INSTANTIATE_FWD(f16_t, 128, false)
+DK_INSTANTIATE_FWD(f16_t, 64, false)
+DK_INSTANTIATE_FWD(bf16_t, 128, true)
+DK_INSTANTIATE_FWD(bf16_t, 64, true)
+DK_INSTANTIATE_FWD(f16_t, 128, true)
+DK_INSTANTIATE_FWD(f16_t, 64, true)
 #undef DK_INSTANTIATE_FWD
 
 // Largest G in {4, 2, 1} such that G consecutive q heads share the kv head and
@@ -532,16 +546,16 @@ static int fwd_group(const FwdParams &p) {
 }
 
 bool mfma_fwd_supported(const FwdParams &p, int dtype) {
-  return (dtype == DK_BF16 || dtype == DK_F16) && (p.D == 128 || p.D == 64) && p.csr.block_rows == 64 &&
+  return (dtype == DK_BF16 || dtype == DK_F16) && mfma_head_dim_ok(p.D) && p.csr.block_rows == 64 &&
          p.csr.block_cols == 64 && p.csr.entry_width == 1 && p.vec_ok;
 }
 
-template <typename T, int D, int G>
+template <typename T, int D, int G, bool PAD>
 static int launch_tdg(const FwdParams &p, dim3 grid, int tiles_y, hipStream_t stream) {
   constexpr int smem = 2 * FwdSmem<D>::kStage;
   static bool attr_set = false;  // raising the dynamic LDS limit is idempotent; a race only repeats it
   if (!attr_set) {
-    DK_HIP_CHECK(hipFuncSetAttribute((const void *)mfma_fwd_kernel<T, D, G>,
+    DK_HIP_CHECK(hipFuncSetAttribute((const void *)mfma_fwd_kernel<T, D, G, PAD>,
                                      hipFuncAttributeMaxDynamicSharedMemorySize, smem));
     attr_set = true;
   }
@@ -554,26 +568,34 @@ static int launch_tdg(const FwdParams &p, dim3 grid, int tiles_y, hipStream_t st
   if constexpr (G == 1) if (pipe) {
     static bool pipe_attr_set = false;
     if (!pipe_attr_set) {
-      DK_HIP_CHECK(hipFuncSetAttribute((const void *)mfma_fwd_pipe_kernel<T, D, G>,
+      DK_HIP_CHECK(hipFuncSetAttribute((const void *)mfma_fwd_pipe_kernel<T, D, G, PAD>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem));
       pipe_attr_set = true;
     }
-    hipLaunchKernelGGL((mfma_fwd_pipe_kernel<T, D, G>), grid, dim3(128 * G), smem, stream, p, tiles_y);
+    hipLaunchKernelGGL((mfma_fwd_pipe_kernel<T, D, G, PAD>), grid, dim3(128 * G), smem, stream, p, tiles_y);
     DK_HIP_CHECK(hipGetLastError());
     return DK_OK;
   }
-  hipLaunchKernelGGL((mfma_fwd_kernel<T, D, G>), grid, dim3(128 * G), smem, stream, p, tiles_y);
+  hipLaunchKernelGGL((mfma_fwd_kernel<T, D, G, PAD>), grid, dim3(128 * G), smem, stream, p, tiles_y);
   DK_HIP_CHECK(hipGetLastError());
   return DK_OK;
 }
 
-template <typename T, int D>
-static int launch_td(const FwdParams &p, dim3 grid, int tiles_y, hipStream_t stream) {
+template <typename T, int D, bool PAD>
+static int launch_tdp(const FwdParams &p, dim3 grid, int tiles_y, hipStream_t stream) {
   switch (fwd_group(p)) {
-    case 4: return launch_tdg<T, D, 4>(p, grid, tiles_y, stream);
-    case 2: return launch_tdg<T, D, 2>(p, grid, tiles_y, stream);
-    default: return launch_tdg<T, D, 1>(p, grid, tiles_y, stream);
+    case 4: return launch_tdg<T, D, 4, PAD>(p, grid, tiles_y, stream);
+    case 2: return launch_tdg<T, D, 2, PAD>(p, grid, tiles_y, stream);
+    default: return launch_tdg<T, D, 1, PAD>(p, grid, tiles_y, stream);
   }
+}
+
+// head dims below the tile width (64 or 128) run the zero-padded instantiation
+template <typename T>
+static int launch_t(const FwdParams &p, dim3 grid, int tiles_y, hipStream_t stream) {
+  if (p.D == 128) return launch_tdp<T, 128, false>(p, grid, tiles_y, stream);
+  if (p.D == 64) return launch_tdp<T, 64, false>(p, grid, tiles_y, stream);
+  return p.D > 64 ? launch_tdp<T, 128, true>(p, grid, tiles_y, stream) : launch_tdp<T, 64, true>(p, grid, tiles_y, stream);
 }
 
 int launch_mfma_fwd(const FwdParams &p, int dtype, hipStream_t stream) {
@@ -589,9 +611,7 @@ int launch_mfma_fwd(const FwdParams &p, int dtype, hipStream_t stream) {
   }
   DK_REQUIRE(tiles <= 65535, "too many q tiles for one launch (%d)", tiles);
   dim3 grid(1, tiles, s.packed ? 1 : s.batch);
-  if (dtype == DK_BF16)
-    return p.D == 128 ? launch_td<bf16_t, 128>(p, grid, tiles, stream) : launch_td<bf16_t, 64>(p, grid, tiles, stream);
-  return p.D == 128 ? launch_td<f16_t, 128>(p, grid, tiles, stream) : launch_td<f16_t, 64>(p, grid, tiles, stream);
+  return dtype == DK_BF16 ? launch_t<bf16_t>(p, grid, tiles, stream) : launch_t<f16_t>(p, grid, tiles, stream);
 }
 
 }  // namespace dk

@@ -102,6 +102,31 @@ def test_dims_not_power_of_two(impl, D, dtype):
     run_fwd_bwd(1, 2, 2, 384, D, dtype, 64, 2, 3, homo_head=(D < 100))
 
 
+@pytest.mark.parametrize("D,dtype", [(96, torch.bfloat16), (48, torch.float16), (80, torch.bfloat16),
+                                     (8, torch.float16), (120, torch.bfloat16)])
+def test_head_dims_below_tile_width(impl, D, dtype):
+    """Head dims that are multiples of 8 below 64 / 128 run the matrix-core kernels zero-padded
+    on chip: GQA group of 4 (shared K/V tiles), MHA (software-pipelined forward), ragged length,
+    blocks of 128 on split tiles, non-causal."""
+    run_fwd_bwd(2, 8, 2, 512, D, dtype, 64, 2, 4)
+    run_fwd_bwd(1, 4, 4, 1000, D, dtype, 64, 3, 3)
+    run_fwd_bwd(1, 4, 2, 777, D, dtype, 128, 1, 2, non_contiguous=True)
+    run_fwd_bwd(1, 2, 2, 512, D, dtype, 64, 2, 4, causal=False)
+
+
+def test_matrix_core_kernels_take_padded_dims_and_split_blocks():
+    """With the implementation forced to the matrix-core kernels (no generic fallback), padded
+    head dims and 128-blocks must run, and a head dim they do not cover must be refused."""
+    ops.set_impl("mfma")
+    try:
+        run_fwd_bwd(1, 8, 2, 512, 96, torch.bfloat16, 64, 2, 4)
+        run_fwd_bwd(1, 4, 4, 512, 48, torch.float16, 128, 1, 2)
+        with pytest.raises(Exception, match="no MFMA"):
+            run_fwd_bwd(1, 2, 2, 256, 160, torch.bfloat16, 64, 2, 4)
+    finally:
+        ops.set_impl("auto")
+
+
 @pytest.mark.parametrize("L", [15, 100, 1028, 777])
 def test_ragged_lengths(impl, L):
     run_fwd_bwd(2, 4, 4, L, 128, torch.bfloat16, 64 if L != 1028 else 32, 2, 4)
@@ -226,7 +251,16 @@ def test_right_padded_prefill(impl):
                                              (128, None, True)])
 def test_decode(impl, bs, block_m, left):
     """One new token per sequence over left-padded / right-padded / unpadded KV, GQA."""
-    B, Hq, Hkv, Lmax, D = 4, 8, 2, 2048, 128
+    _decode_case(bs, block_m, left, 128)
+
+
+@pytest.mark.parametrize("D,left", [(96, True), (48, False), (120, True)])
+def test_decode_head_dims_below_tile_width(impl, D, left):
+    _decode_case(64, None, left, D)
+
+
+def _decode_case(bs, block_m, left, D):
+    B, Hq, Hkv, Lmax = 4, 8, 2, 2048
     sm = 1 / math.sqrt(D)
     q, k, v = make_qkv(B, 1, Lmax, Hq, Hkv, D, torch.bfloat16, 1)
     lens = [64 * 21 + 12, 2048, 1, 64 * 5]
@@ -254,8 +288,9 @@ def test_decode(impl, bs, block_m, left):
     assert_close("O unpadded", out2[0], ro, **TOL)
 
 
-def test_packed_varlen_prefill_and_decode(impl):
-    Hq, Hkv, D, bs = 4, 2, 128, 32
+@pytest.mark.parametrize("D,bs", [(128, 32), (96, 64), (128, 128)])
+def test_packed_varlen_prefill_and_decode(impl, D, bs):
+    Hq, Hkv = 4, 2
     sm = 1 / math.sqrt(D)
     lens = [300, 1, 64, 517, 129]
     T = sum(lens)

@@ -52,7 +52,8 @@ class BwdArgs(C.Structure):
                 ("lse", RowVec), ("dlse", RowVec), ("delta", vp),
                 ("csr", Lut), ("csc", Lut), ("seqs", Seqs),
                 ("num_q_heads", i32), ("num_kv_heads", i32), ("head_dim", i32),
-                ("dtype", i32), ("causal", i32), ("impl", i32), ("sm_scale", f32), ("stream", vp)]
+                ("dtype", i32), ("causal", i32), ("impl", i32), ("sm_scale", f32),
+                ("workspace", vp), ("workspace_bytes", C.c_size_t), ("stream", vp)]
 
 
 # name -> (restype, argtypes); every symbol include/dkernel_hip.h declares
@@ -68,6 +69,7 @@ SYMBOLS = {
     "dk_fwd": (C.c_int, [C.POINTER(FwdArgs)]),
     "dk_fwd_workspace_bytes": (C.c_size_t, [C.POINTER(FwdArgs)]),
     "dk_bwd": (C.c_int, [C.POINTER(BwdArgs)]),
+    "dk_bwd_workspace_bytes": (C.c_size_t, [C.POINTER(BwdArgs)]),
 }
 
 _lib = None

@@ -14,7 +14,8 @@ int launch_generic_bwd(const BwdParams &p, int dtype, hipStream_t stream);
 bool mfma_fwd_supported(const FwdParams &p, int dtype);
 int launch_mfma_fwd(const FwdParams &p, int dtype, hipStream_t stream);
 bool mfma_bwd_supported(const BwdParams &p, int dtype);
-int launch_mfma_bwd(const BwdParams &p, int dtype, hipStream_t stream);
+int launch_mfma_bwd(const BwdParams &p, int dtype, void *workspace, size_t workspace_bytes, hipStream_t stream);
+size_t mfma_bwd_workspace_bytes(const BwdParams &p);
 bool decode_supported(const FwdParams &p, int dtype);
 size_t decode_workspace_bytes(const FwdParams &p);
 int launch_decode(const FwdParams &p, int dtype, void *workspace, size_t workspace_bytes, hipStream_t stream);
@@ -95,6 +96,55 @@ static int make_fwd_params(const dk_fwd_args *a, FwdParams &p) {
   return DK_OK;
 }
 
+// Checks the backward arguments and fills the kernel parameter block.  `empty` is set when
+// there is nothing to compute (no pointers are looked at then).
+static int make_bwd_params(const dk_bwd_args *a, BwdParams &p, bool &empty) {
+  empty = false;
+  DK_REQUIRE(a != nullptr, "args is NULL");
+  int rc = check_common(a->seqs, a->num_q_heads, a->num_kv_heads, a->head_dim, a->dtype, a->causal);
+  if (rc) return rc;
+  DK_REQUIRE(!a->seqs.q_starts && !a->seqs.packed,
+             "Currently does not support paddings or variable length inputs in backward.");
+  rc = check_lut(a->csr, "csr", a->num_q_heads, a->num_kv_heads);
+  if (rc) return rc;
+  rc = check_lut(a->csc, "csc", a->num_q_heads, a->num_kv_heads);
+  if (rc) return rc;
+  DK_REQUIRE(a->csc.entry_width == 1, "csc table cannot carry values");
+  DK_REQUIRE((int64_t)a->csr.num_rows * a->csr.block_rows >= a->seqs.max_k_len,
+             "Input length %d is larger than the maximum length allowed", a->seqs.max_k_len);
+  if (a->seqs.batch == 0 || a->seqs.max_q_len == 0) {
+    empty = true;
+    return DK_OK;
+  }
+  DK_REQUIRE(a->q.ptr && a->k.ptr && a->v.ptr && a->o.ptr && a->dout.ptr && a->dq.ptr && a->dk.ptr && a->dv.ptr,
+             "a tensor pointer is NULL");
+  DK_REQUIRE(a->lse.ptr && a->delta, "lse / delta is NULL");
+  p.q = view(a->q);
+  p.k = view(a->k);
+  p.v = view(a->v);
+  p.o = view(a->o);
+  p.dout = view(a->dout);
+  p.dq = view(a->dq);
+  p.dk = view(a->dk);
+  p.dv = view(a->dv);
+  p.lse = view(a->lse);
+  p.dlse = view(a->dlse);
+  p.delta = a->delta;
+  p.csr = view(a->csr);
+  p.csc = view(a->csc);
+  p.seqs = view(a->seqs);
+  p.Hq = a->num_q_heads;
+  p.Hkv = a->num_kv_heads;
+  p.D = a->head_dim;
+  p.causal = a->causal ? 1 : 0;
+  p.sm_scale = a->sm_scale;
+  p.scale_log2 = a->sm_scale * kLog2e;
+  const size_t es = elem_size(a->dtype);
+  p.vec_ok = vec_aligned(a->q, es) && vec_aligned(a->k, es) && vec_aligned(a->v, es) && vec_aligned(a->o, es) &&
+             vec_aligned(a->dout, es) && vec_aligned(a->dq, es) && vec_aligned(a->dk, es) && vec_aligned(a->dv, es);
+  return DK_OK;
+}
+
 }  // namespace dk
 
 using namespace dk;
@@ -127,52 +177,24 @@ int dk_fwd(const dk_fwd_args *a) {
   return launch_generic_fwd(p, a->dtype, stream);
 }
 
+size_t dk_bwd_workspace_bytes(const dk_bwd_args *a) {
+  BwdParams p;
+  bool empty;
+  if (make_bwd_params(a, p, empty) != DK_OK || empty) return 0;
+  if (a->impl != DK_IMPL_GENERIC && mfma_bwd_supported(p, a->dtype)) return mfma_bwd_workspace_bytes(p);
+  return 0;
+}
+
 int dk_bwd(const dk_bwd_args *a) {
   clear_error();
-  DK_REQUIRE(a != nullptr, "args is NULL");
-  int rc = check_common(a->seqs, a->num_q_heads, a->num_kv_heads, a->head_dim, a->dtype, a->causal);
-  if (rc) return rc;
-  DK_REQUIRE(!a->seqs.q_starts && !a->seqs.packed,
-             "Currently does not support paddings or variable length inputs in backward.");
-  rc = check_lut(a->csr, "csr", a->num_q_heads, a->num_kv_heads);
-  if (rc) return rc;
-  rc = check_lut(a->csc, "csc", a->num_q_heads, a->num_kv_heads);
-  if (rc) return rc;
-  DK_REQUIRE(a->csc.entry_width == 1, "csc table cannot carry values");
-  DK_REQUIRE((int64_t)a->csr.num_rows * a->csr.block_rows >= a->seqs.max_k_len,
-             "Input length %d is larger than the maximum length allowed", a->seqs.max_k_len);
-  if (a->seqs.batch == 0 || a->seqs.max_q_len == 0) return DK_OK;
-  DK_REQUIRE(a->q.ptr && a->k.ptr && a->v.ptr && a->o.ptr && a->dout.ptr && a->dq.ptr && a->dk.ptr && a->dv.ptr,
-             "a tensor pointer is NULL");
-  DK_REQUIRE(a->lse.ptr && a->delta, "lse / delta is NULL");
   BwdParams p;
-  p.q = view(a->q);
-  p.k = view(a->k);
-  p.v = view(a->v);
-  p.o = view(a->o);
-  p.dout = view(a->dout);
-  p.dq = view(a->dq);
-  p.dk = view(a->dk);
-  p.dv = view(a->dv);
-  p.lse = view(a->lse);
-  p.dlse = view(a->dlse);
-  p.delta = a->delta;
-  p.csr = view(a->csr);
-  p.csc = view(a->csc);
-  p.seqs = view(a->seqs);
-  p.Hq = a->num_q_heads;
-  p.Hkv = a->num_kv_heads;
-  p.D = a->head_dim;
-  p.causal = a->causal ? 1 : 0;
-  p.sm_scale = a->sm_scale;
-  p.scale_log2 = a->sm_scale * kLog2e;
-  const size_t es = elem_size(a->dtype);
-  p.vec_ok = vec_aligned(a->q, es) && vec_aligned(a->k, es) && vec_aligned(a->v, es) && vec_aligned(a->o, es) &&
-             vec_aligned(a->dout, es) && vec_aligned(a->dq, es) && vec_aligned(a->dk, es) && vec_aligned(a->dv, es);
+  bool empty;
+  const int rc = make_bwd_params(a, p, empty);
+  if (rc || empty) return rc;
   hipStream_t stream = (hipStream_t)a->stream;
   if (a->impl != DK_IMPL_GENERIC) {
     if (mfma_bwd_supported(p, a->dtype)) {
-      return launch_mfma_bwd(p, a->dtype, stream);
+      return launch_mfma_bwd(p, a->dtype, a->workspace, a->workspace_bytes, stream);
     }
     if (a->impl == DK_IMPL_MFMA)
       return fail(DK_ERR_UNSUPPORTED, "no MFMA backward kernel for dtype %d, head_dim %d, tiles (%d, %d)",

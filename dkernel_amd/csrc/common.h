@@ -28,6 +28,7 @@ void clear_error();
   } while (0)
 
 inline int cdiv(int a, int b) { return (a + b - 1) / b; }
+inline int64_t cdiv64(int64_t a, int64_t b) { return (a + b - 1) / b; }
 inline bool is_pow2(int x) { return x > 0 && (x & (x - 1)) == 0; }
 
 }  // namespace dk

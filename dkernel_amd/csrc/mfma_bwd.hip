@@ -291,7 +291,7 @@ struct DkdvSmem {
 };
 
 template <typename T, int D, bool PAD>
-__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void mfma_dkdv_kernel(const BwdParams p) {
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void mfma_dkdv_kernel(const BwdParams p, int head_split) {
   using M = Mma<T>;
   using vec8 = typename M::vec8;
   using TL = Tile<D>;
@@ -304,8 +304,13 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const SeqInfo sq = load_seq(p.seqs, blockIdx.z, p.causal);
   const int cb = blockIdx.y;
   if (cb * 64 >= sq.k_len) return;
-  const int kvh = blockIdx.x;
+  // head_split: one workgroup per q head instead of per kv head; p.dk / p.dv then describe
+  // per-q-head partial buffers that a second kernel sums over each kv group
   const int ratio = __builtin_amdgcn_readfirstlane(p.Hq / p.Hkv);  // integer division runs on the VALU
+  const int out_head = blockIdx.x;
+  const int kvh = head_split ? __builtin_amdgcn_readfirstlane(out_head / ratio) : out_head;
+  const int gq_first = head_split ? out_head - kvh * ratio : 0;
+  const int gq_end = head_split ? gq_first + 1 : ratio;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int pair = wave & 3, nh = wave & 1, mh = (wave >> 1) & 1;
@@ -345,7 +350,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   transposed_offsets<D>(lane, tr);
   float *xbuf = reinterpret_cast<float *>(smem + S::kX) + pair * 2 * 1024;  // this pair's two P buffers
 
-  for (int gq = 0; gq < ratio; ++gq) {
+  for (int gq = gq_first; gq < gq_end; ++gq) {
     const int h = kvh * ratio + gq;
     const int lh = lut_head(p.csc, h, p.Hq, p.Hkv);
     int e0 = 0, e1 = 0;
@@ -549,8 +554,24 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   __syncthreads();
   if (mh == 1 || !key_ok) return;
   const float out_scale = dp_wave ? p.sm_scale : 1.f;
-  T *outp = dp_wave ? (T *)p.dk.ptr + sq.b * p.dk.sb + kvh * p.dk.sh + (int64_t)key * p.dk.st
-                    : (T *)p.dv.ptr + sq.b * p.dv.sb + kvh * p.dv.sh + (int64_t)key * p.dv.st;
+  const TensorView &outv = dp_wave ? p.dk : p.dv;
+  const int64_t out_off = sq.b * outv.sb + out_head * outv.sh + (int64_t)key * outv.st;
+  if (head_split) {  // fp32 partial of this q head
+    float *outp = (float *)outv.ptr + out_off;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) {
+        float4 o4;
+        o4.x = (acc[dt][r4 * 4 + 0] + red[(dt * 16 + r4 * 4 + 0) * 64 + lane]) * out_scale;
+        o4.y = (acc[dt][r4 * 4 + 1] + red[(dt * 16 + r4 * 4 + 1) * 64 + lane]) * out_scale;
+        o4.z = (acc[dt][r4 * 4 + 2] + red[(dt * 16 + r4 * 4 + 2) * 64 + lane]) * out_scale;
+        o4.w = (acc[dt][r4 * 4 + 3] + red[(dt * 16 + r4 * 4 + 3) * 64 + lane]) * out_scale;
+        if (!PAD || dt * 32 + r4 * 8 + g * 4 < p.D) *reinterpret_cast<float4 *>(outp + dt * 32 + r4 * 8 + g * 4) = o4;
+      }
+    return;
+  }
+  T *outp = (T *)outv.ptr + out_off;
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -576,14 +597,54 @@ template __global__ void mfma_dq_kernel<f16_t, 128, false>(const BwdParams, int)
 template __global__ void mfma_dq_kernel<f16_t, 128, true>(const BwdParams, int);
 template __global__ void mfma_dq_kernel<f16_t, 64, false>(const BwdParams, int);
 template __global__ void mfma_dq_kernel<f16_t, 64, true>(const BwdParams, int);
-template __global__ void mfma_dkdv_kernel<bf16_t, 128, false>(const BwdParams);
-template __global__ void mfma_dkdv_kernel<bf16_t, 128, true>(const BwdParams);
-template __global__ void mfma_dkdv_kernel<bf16_t, 64, false>(const BwdParams);
-template __global__ void mfma_dkdv_kernel<bf16_t, 64, true>(const BwdParams);
-template __global__ void mfma_dkdv_kernel<f16_t, 128, false>(const BwdParams);
-template __global__ void mfma_dkdv_kernel<f16_t, 128, true>(const BwdParams);
-template __global__ void mfma_dkdv_kernel<f16_t, 64, false>(const BwdParams);
-template __global__ void mfma_dkdv_kernel<f16_t, 64, true>(const BwdParams);
+template __global__ void mfma_dkdv_kernel<bf16_t, 128, false>(const BwdParams, int);
+template __global__ void mfma_dkdv_kernel<bf16_t, 128, true>(const BwdParams, int);
+template __global__ void mfma_dkdv_kernel<bf16_t, 64, false>(const BwdParams, int);
+template __global__ void mfma_dkdv_kernel<bf16_t, 64, true>(const BwdParams, int);
+template __global__ void mfma_dkdv_kernel<f16_t, 128, false>(const BwdParams, int);
+template __global__ void mfma_dkdv_kernel<f16_t, 128, true>(const BwdParams, int);
+template __global__ void mfma_dkdv_kernel<f16_t, 64, false>(const BwdParams, int);
+template __global__ void mfma_dkdv_kernel<f16_t, 64, true>(const BwdParams, int);
+
+// Sum of the per-q-head dK / dV partials over each kv group (head_split mode).  One thread
+// per 8 head dims of one (batch, kv head, key): blockIdx.y = 0 sums dK, 1 sums dV.
+// part: fp32 [batch][Hq][keys][D] contiguous.
+template <typename T>
+__global__ __launch_bounds__(256) void dkdv_group_sum_kernel(const float *part_k, const float *part_v, TensorView dk,
+                                                             TensorView dv, int batch, int Hq, int Hkv, int keys,
+                                                             int D) {
+  const int cpr = D / 8;
+  const int64_t total = (int64_t)batch * Hkv * keys * cpr;
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const int ch = (int)(i % cpr);
+  const int key = (int)((i / cpr) % keys);
+  const int kvh = (int)((i / ((int64_t)cpr * keys)) % Hkv);
+  const int b = (int)(i / ((int64_t)cpr * keys * Hkv));
+  const int ratio = Hq / Hkv;
+  const float *part = blockIdx.y ? part_v : part_k;
+  const TensorView &out = blockIdx.y ? dv : dk;
+  float4 lo = make_float4(0.f, 0.f, 0.f, 0.f), hi = lo;
+  const float *src = part + (((int64_t)b * Hq + kvh * ratio) * keys + key) * D + ch * 8;
+  for (int gq = 0; gq < ratio; ++gq) {
+    const float4 a = *reinterpret_cast<const float4 *>(src + (int64_t)gq * keys * D);
+    const float4 c = *reinterpret_cast<const float4 *>(src + (int64_t)gq * keys * D + 4);
+    lo.x += a.x, lo.y += a.y, lo.z += a.z, lo.w += a.w;
+    hi.x += c.x, hi.y += c.y, hi.z += c.z, hi.w += c.w;
+  }
+  T o8[8] = {from_float<T>(lo.x), from_float<T>(lo.y), from_float<T>(lo.z), from_float<T>(lo.w),
+             from_float<T>(hi.x), from_float<T>(hi.y), from_float<T>(hi.z), from_float<T>(hi.w)};
+  *reinterpret_cast<uint4 *>((T *)out.ptr + b * out.sb + kvh * out.sh + (int64_t)key * out.st + ch * 8) =
+      *reinterpret_cast<const uint4 *>(o8);
+}
+
+// Scratch for the head-split dK/dV pass: fp32 per-q-head partials of dK and dV (16-bit partials
+// would round each head's share before the sum).  Zero when the pass would not be split (one
+// q head per kv head).
+size_t mfma_bwd_workspace_bytes(const BwdParams &p) {
+  if (p.Hq == p.Hkv) return 0;
+  return 2 * (size_t)p.seqs.batch * p.Hq * p.seqs.max_k_len * p.D * sizeof(float);
+}
 
 bool mfma_bwd_supported(const BwdParams &p, int dtype) {
   return (dtype == DK_BF16 || dtype == DK_F16) && mfma_head_dim_ok(p.D) && p.csr.block_rows == 64 &&
@@ -592,7 +653,7 @@ bool mfma_bwd_supported(const BwdParams &p, int dtype) {
 }
 
 template <typename T, int D, bool PAD>
-static int launch_bwd_td(const BwdParams &p, hipStream_t stream) {
+static int launch_bwd_td(const BwdParams &p, void *workspace, size_t workspace_bytes, hipStream_t stream) {
   const SeqView &s = p.seqs;
   constexpr int smem_dq = 2 * 2 * Tile<D>::kBytes;
   constexpr int smem_dkdv = DkdvSmem<D>::kBytes;
@@ -611,21 +672,42 @@ static int launch_bwd_td(const BwdParams &p, hipStream_t stream) {
   // dQ first: it also writes delta, which the dK/dV pass reads
   hipLaunchKernelGGL((mfma_dq_kernel<T, D, PAD>), dim3(p.Hq, tiles, s.batch), dim3(256), smem_dq, stream, p, tiles);
   DK_HIP_CHECK(hipGetLastError());
-  hipLaunchKernelGGL((mfma_dkdv_kernel<T, D, PAD>), dim3(p.Hkv, cblocks, s.batch), dim3(512), smem_dkdv, stream, p);
+  // With several q heads per kv head a workgroup per kv head walks all of them, and the longest
+  // column (a vertical one near the start: every later q block, times the group size) alone
+  // outlasts the average CU's share of the whole pass.  Given scratch, the pass runs one
+  // workgroup per q head into per-head partials and a bandwidth-bound kernel sums each group.
+  const size_t need = mfma_bwd_workspace_bytes(p);
+  if (need > 0 && workspace && workspace_bytes >= need && ((uintptr_t)workspace % 16) == 0) {
+    BwdParams pp = p;
+    const int64_t keys = s.max_k_len;
+    float *part_k = (float *)workspace, *part_v = part_k + (int64_t)s.batch * p.Hq * keys * p.D;
+    pp.dk = TensorView{part_k, p.Hq * keys * p.D, keys * p.D, p.D};
+    pp.dv = TensorView{part_v, p.Hq * keys * p.D, keys * p.D, p.D};
+    hipLaunchKernelGGL((mfma_dkdv_kernel<T, D, PAD>), dim3(p.Hq, cblocks, s.batch), dim3(512), smem_dkdv, stream, pp, 1);
+    DK_HIP_CHECK(hipGetLastError());
+    const int64_t total = (int64_t)s.batch * p.Hkv * keys * (p.D / 8);
+    hipLaunchKernelGGL((dkdv_group_sum_kernel<T>), dim3((unsigned)cdiv64(total, 256), 2), dim3(256), 0, stream, part_k,
+                       part_v, p.dk, p.dv, s.batch, p.Hq, p.Hkv, (int)keys, p.D);
+    DK_HIP_CHECK(hipGetLastError());
+    return DK_OK;
+  }
+  hipLaunchKernelGGL((mfma_dkdv_kernel<T, D, PAD>), dim3(p.Hkv, cblocks, s.batch), dim3(512), smem_dkdv, stream, p, 0);
   DK_HIP_CHECK(hipGetLastError());
   return DK_OK;
 }
 
 // head dims below the tile width (64 or 128) run the zero-padded instantiation
 template <typename T>
-static int launch_bwd_t(const BwdParams &p, hipStream_t stream) {
-  if (p.D == 128) return launch_bwd_td<T, 128, false>(p, stream);
-  if (p.D == 64) return launch_bwd_td<T, 64, false>(p, stream);
-  return p.D > 64 ? launch_bwd_td<T, 128, true>(p, stream) : launch_bwd_td<T, 64, true>(p, stream);
+static int launch_bwd_t(const BwdParams &p, void *ws, size_t ws_bytes, hipStream_t stream) {
+  if (p.D == 128) return launch_bwd_td<T, 128, false>(p, ws, ws_bytes, stream);
+  if (p.D == 64) return launch_bwd_td<T, 64, false>(p, ws, ws_bytes, stream);
+  return p.D > 64 ? launch_bwd_td<T, 128, true>(p, ws, ws_bytes, stream)
+                  : launch_bwd_td<T, 64, true>(p, ws, ws_bytes, stream);
 }
 
-int launch_mfma_bwd(const BwdParams &p, int dtype, hipStream_t stream) {
-  return dtype == DK_BF16 ? launch_bwd_t<bf16_t>(p, stream) : launch_bwd_t<f16_t>(p, stream);
+int launch_mfma_bwd(const BwdParams &p, int dtype, void *workspace, size_t workspace_bytes, hipStream_t stream) {
+  return dtype == DK_BF16 ? launch_bwd_t<bf16_t>(p, workspace, workspace_bytes, stream)
+                          : launch_bwd_t<f16_t>(p, workspace, workspace_bytes, stream);
 }
 
 }  // namespace dk

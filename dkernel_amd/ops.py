@@ -27,6 +27,9 @@ _IMPL = {"auto": _lib.DK_IMPL_AUTO, "generic": _lib.DK_IMPL_GENERIC, "mfma": _li
 _impl = _lib.DK_IMPL_AUTO
 
 
+_bwd_workspace = True  # hand dk_bwd the scratch it asks for (off: tests of the path without it)
+
+
 def set_impl(name: str) -> None:
     global _impl
     _impl = _IMPL[name]
@@ -200,7 +203,12 @@ def _backward(ctx, do: Tensor, dlse: Optional[Tensor],
     args.dtype, args.causal, args.impl = _DTYPES[q.dtype], int(bool(ctx.causal)), _impl
     args.sm_scale = float(ctx.sm_scale)
     args.stream = _stream()
-    _lib.check(_lib.lib().dk_bwd(C.byref(args)))
+    lib = _lib.lib()
+    need = lib.dk_bwd_workspace_bytes(C.byref(args)) if _bwd_workspace else 0
+    if need:  # per-q-head dK/dV partials of the head-split pass (several q heads per kv head)
+        ws = torch.empty(need, dtype=torch.uint8, device=q.device)
+        args.workspace, args.workspace_bytes = ws.data_ptr(), need
+    _lib.check(lib.dk_bwd(C.byref(args)))
     return dq, dk, dv
 
 

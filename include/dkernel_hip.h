@@ -156,8 +156,12 @@ size_t dk_fwd_workspace_bytes(const dk_fwd_args *args);
 /* Backward of dk_fwd for equal-length, unpadded sequences (seqs pointers
  * NULL).  delta is caller scratch of batch * num_q_heads * max_q_len floats.
  * dlse.ptr may be NULL.  dk/dv are written for every kv head (sum over the q
- * heads of the group).  Replaces _bwd_preprocess and _sparse_bwd_kernel
- * launches, dkernel/ops/sparse_attn_bwd.py:781-788, :811-850. */
+ * heads of the group).  workspace is optional device scratch (16-byte
+ * aligned, dk_bwd_workspace_bytes): with it and several q heads per kv head
+ * the dK/dV pass runs one workgroup per q head and sums the groups afterwards,
+ * which balances much better; without it the result is the same, only
+ * slower.  Replaces _bwd_preprocess and _sparse_bwd_kernel launches,
+ * dkernel/ops/sparse_attn_bwd.py:781-788, :811-850. */
 typedef struct dk_bwd_args {
   dk_tensor q, k, v, o, dout, dq, dk, dv;
   dk_rowvec lse, dlse;
@@ -169,10 +173,14 @@ typedef struct dk_bwd_args {
   int32_t causal;
   int32_t impl;
   float sm_scale;
+  void *workspace;        /* optional device scratch, may be NULL */
+  size_t workspace_bytes;
   void *stream;
 } dk_bwd_args;
 
 int dk_bwd(const dk_bwd_args *args);
+/* Scratch that dk_bwd can use for these arguments (0 = none useful). */
+size_t dk_bwd_workspace_bytes(const dk_bwd_args *args);
 
 #ifdef __cplusplus
 }

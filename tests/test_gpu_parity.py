@@ -136,6 +136,16 @@ def test_gqa(impl):
     run_fwd_bwd(2, 8, 2, 512, 128, torch.bfloat16, 64, 3, 4)
 
 
+def test_gqa_backward_with_and_without_scratch(monkeypatch):
+    """dk_bwd sums dK/dV over a kv group either inside one workgroup (no scratch) or from
+    per-q-head partials (scratch given): both must meet the oracle, for plain and padded dims."""
+    for use in (True, False):
+        monkeypatch.setattr(ops, "_bwd_workspace", use)
+        run_fwd_bwd(2, 8, 2, 1024, 128, torch.bfloat16, 64, 3, 4)
+        run_fwd_bwd(1, 6, 2, 777, 96, torch.float16, 64, 2, 3)
+        run_fwd_bwd(1, 8, 1, 512, 64, torch.bfloat16, 64, 2, 4, seq_dim=2, non_contiguous=True)
+
+
 def test_patterns(impl):
     run_fwd_bwd(1, 8, 8, 1024, 128, torch.bfloat16, 64, 10, 3)
     run_fwd_bwd(1, 8, 8, 1024, 128, torch.bfloat16, 64, 1, 8)

@@ -26,7 +26,7 @@ def test_library_exports_every_declared_symbol():
     handle = ctypes.CDLL(_lib.LIB_PATH)
     for name in declared:
         assert hasattr(handle, name), name
-    assert _lib.lib().dk_version() >= 100
+    assert _lib.lib().dk_version() >= 200
     assert _lib.lib().dk_last_error() is not None
 
 
@@ -35,7 +35,7 @@ def test_struct_sizes_match_header():
     assert ctypes.sizeof(_lib.Tensor) == 32 and ctypes.sizeof(_lib.RowVec) == 32
     assert ctypes.sizeof(_lib.Lut) == 64 and ctypes.sizeof(_lib.Seqs) == 48
     assert ctypes.sizeof(_lib.FwdArgs) == 4 * 32 + 32 + 64 + 48 + 7 * 4 + 4 + 3 * 8
-    assert ctypes.sizeof(_lib.BwdArgs) == 8 * 32 + 2 * 32 + 8 + 2 * 64 + 48 + 7 * 4 + 4 + 8
+    assert ctypes.sizeof(_lib.BwdArgs) == 8 * 32 + 2 * 32 + 8 + 2 * 64 + 48 + 7 * 4 + 4 + 3 * 8
 
 
 def test_mask_and_luts_match_fixtures(lut_fixtures):

@@ -102,9 +102,14 @@ def _stream() -> C.c_void_p:
     return C.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
+last_fwd_workspace_bytes = 0  # scratch the library asked for in the latest forward (non-zero: split-KV decode)
+
+
 def _run_fwd(args: _lib.FwdArgs, device) -> None:
+    global last_fwd_workspace_bytes
     lib = _lib.lib()
     need = lib.dk_fwd_workspace_bytes(C.byref(args))
+    last_fwd_workspace_bytes = need
     ws = None
     if need:
         ws = torch.empty(need, dtype=torch.uint8, device=device)
@@ -308,9 +313,11 @@ def varlen_sparse_attn(q: Tensor, k: Tensor, v: Tensor,
     assert k.shape == v.shape
     assert cu_seqlens_k.dim() == 1
     dev = q.device
+    single_query = False
     if cu_seqlens_q is None:
         if q.size(0) == batch_size:  # decoding only
             cu_seqlens_q = torch.arange(0, batch_size + 1, dtype=torch.int32, device=dev)
+            single_query = True  # lets the library take the split-KV decode kernel
         elif q.size(0) == k.size(0):
             cu_seqlens_q = cu_seqlens_k
         else:
@@ -328,7 +335,7 @@ def varlen_sparse_attn(q: Tensor, k: Tensor, v: Tensor,
     args.lse = _rowvec(lse, (0, lse.stride(0), lse.stride(1))) if lse is not None else _rowvec(None)
     args.csr = _lut(sparse_layout, dev, lut_group)
     isz = cu_q.element_size()
-    args.seqs = _lib.Seqs(batch_size, q.size(0), k.size(0), 1,
+    args.seqs = _lib.Seqs(batch_size, q.size(0), k.size(0), 3 if single_query else 1,
                           cu_q.data_ptr(), cu_q.data_ptr() + isz, cu_k.data_ptr(), cu_k.data_ptr() + isz)
     args.num_q_heads, args.num_kv_heads, args.head_dim = num_heads, k.size(1), head_size
     args.dtype, args.causal, args.impl = _DTYPES[q.dtype], int(bool(causal)), _impl

@@ -124,7 +124,9 @@ typedef struct dk_seqs {
   int32_t batch;
   int32_t max_q_len; /* extent of the q token dimension (total tokens when packed) */
   int32_t max_k_len;
-  int32_t packed;    /* 1: sequences share one token dimension (3-D inputs) */
+  int32_t packed;    /* bit 0: sequences share one token dimension (3-D inputs);
+                        bit 1 (with bit 0): the caller guarantees exactly one query token per
+                        sequence, which lets dk_fwd take the split-KV decode path */
   const int32_t *q_starts, *q_ends, *k_starts, *k_ends;
 } dk_seqs;
 

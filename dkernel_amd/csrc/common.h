@@ -2,6 +2,7 @@
 // never lets a C++ exception cross the C ABI, and small host helpers.
 #pragma once
 
+#include <atomic>
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
@@ -25,6 +26,21 @@ void clear_error();
     hipError_t e_ = (expr);                                                             \
     if (e_ != hipSuccess)                                                               \
       return ::dk::fail(DK_ERR_HIP, "%s failed: %s", #expr, hipGetErrorString(e_));     \
+  } while (0)
+
+// Raises a kernel's dynamic LDS limit once per device: the attribute belongs to the current
+// device's copy of the kernel, so a process that uses several GPUs has to set it on each.
+// `done` holds one bit per device ordinal; a race between threads only repeats the call.
+#define DK_ALLOW_DYNAMIC_LDS(kernel, bytes)                                                          \
+  do {                                                                                               \
+    static std::atomic<uint64_t> done_{0};                                                           \
+    int dev_ = 0;                                                                                    \
+    DK_HIP_CHECK(hipGetDevice(&dev_));                                                               \
+    const uint64_t bit_ = 1ull << (dev_ & 63);                                                       \
+    if (!(done_.load(std::memory_order_relaxed) & bit_)) {                                           \
+      DK_HIP_CHECK(hipFuncSetAttribute((const void *)(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (bytes))); \
+      done_.fetch_or(bit_, std::memory_order_relaxed);                                               \
+    }                                                                                                \
   } while (0)
 
 inline int cdiv(int a, int b) { return (a + b - 1) / b; }

@@ -657,14 +657,8 @@ static int launch_bwd_td(const BwdParams &p, void *workspace, size_t workspace_b
   const SeqView &s = p.seqs;
   constexpr int smem_dq = 2 * 2 * Tile<D>::kBytes;
   constexpr int smem_dkdv = DkdvSmem<D>::kBytes;
-  static bool attr_set = false;
-  if (!attr_set) {
-    DK_HIP_CHECK(hipFuncSetAttribute((const void *)mfma_dq_kernel<T, D, PAD>,
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, smem_dq));
-    DK_HIP_CHECK(hipFuncSetAttribute((const void *)mfma_dkdv_kernel<T, D, PAD>,
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, smem_dkdv));
-    attr_set = true;
-  }
+  DK_ALLOW_DYNAMIC_LDS((mfma_dq_kernel<T, D, PAD>), smem_dq);
+  DK_ALLOW_DYNAMIC_LDS((mfma_dkdv_kernel<T, D, PAD>), smem_dkdv);
   const int past = p.causal ? s.max_k_len - s.max_q_len : 0;
   const int tiles = (past + s.max_q_len - 1) / 64 - past / 64 + 1;
   const int cblocks = cdiv(s.max_k_len, 64);

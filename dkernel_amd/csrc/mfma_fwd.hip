@@ -37,7 +37,7 @@ struct FwdSmem {  // one stage = K tile + V tile, swizzled row-major (mfma_commo
   static constexpr int kStage = 2 * Tile<D>::kBytes;
 };
 
-template <typename T, int D, int G, bool PAD>
+template <typename T, int D, int G, bool PAD, bool RP>
 __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 ? 1 : 2, 2))) void mfma_fwd_kernel(const FwdParams p, int tiles_y) {
   using M = Mma<T>;
   using vec8 = typename M::vec8;
@@ -48,17 +48,31 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
   using TL = Tile<D>;
   extern __shared__ __align__(16) char smem[];
 
+  static_assert(!RP || G == 2, "row pairs: two wave pairs, one q tile each");
   SeqInfo sq;
   int tile;
-  const int ty = p.seqs.packed ? blockIdx.y : tiles_y - 1 - (int)blockIdx.y;
-  if (!resolve_tile(p.seqs, p.causal, 64, 1, ty, blockIdx.z, sq, tile)) return;
-  const int rb = sq.past / 64 + tile;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  int rb;
+  int first_rb = 0, last_rb = 0;  // RP: table rows that hold queries of this sequence
+  if constexpr (RP) {
+    // workgroup = table rows 2u and 2u + 1 of one head (one per wave pair); tiles_y counts pairs
+    sq = load_seq(p.seqs, blockIdx.z, p.causal);
+    if (sq.q_len <= 0) return;
+    first_rb = sq.past / 64, last_rb = (sq.past + sq.q_len - 1) / 64;
+    const int u = (first_rb >> 1) + tiles_y - 1 - (int)blockIdx.y;
+    if (u > (last_rb >> 1)) return;
+    rb = 2 * u + (wave >> 1);
+    tile = rb - first_rb;  // outside [0, last_rb - first_rb]: this wave pair has no rows (row_ok false everywhere)
+  } else {
+    const int ty = p.seqs.packed ? blockIdx.y : tiles_y - 1 - (int)blockIdx.y;
+    if (!resolve_tile(p.seqs, p.causal, 64, 1, ty, blockIdx.z, sq, tile)) return;
+    rb = sq.past / 64 + tile;
+  }
   if constexpr (PAD) {  // the slots of the head dims beyond p.D stay zero for the whole kernel
     zero_tiles<NT>(smem, 2 * S::kStage, tid);
     __syncthreads();
   }
-  const int h = blockIdx.x * G + (wave >> 1);
+  const int h = RP ? blockIdx.x : blockIdx.x * G + (wave >> 1);
   const int kvh = __builtin_amdgcn_readfirstlane(h / (p.Hq / p.Hkv));  // integer division runs on the VALU
   const int m = lane & 31, g = lane >> 5;
   const int row0 = rb * 64 + (wave & 1) * 32;  // first absolute position of this wave
@@ -78,9 +92,18 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
     }
   }
 
-  const int lh = lut_head(p.csr, blockIdx.x * G, p.Hq, p.Hkv);
+  const int lh = lut_head(p.csr, RP ? blockIdx.x : blockIdx.x * G, p.Hq, p.Hkv);
   int e0 = 0, e1 = 0;
-  if (rb < p.csr.num_rows) {  // table reads go through the scalar unit (no vector-memory wait)
+  int emid = 0;  // RP: entries [e0, emid) are row 2u, [emid, e1) row 2u + 1 (consecutive rows follow each other)
+  if constexpr (RP) {
+    const int32_t *rp = p.csr.ptr + lh * p.csr.ptr_sh;
+    const int ra = rb & ~1;
+    if (ra < p.csr.num_rows) scalar_load2(rp + ra, rp + ra + 1, e0, emid);
+    e1 = emid;
+    if (ra + 1 < p.csr.num_rows) e1 = scalar_load(rp + ra + 2);
+    if (ra < first_rb) e0 = emid;     // a row without queries of this sequence contributes nothing
+    if (ra + 1 > last_rb) e1 = emid;
+  } else if (rb < p.csr.num_rows) {  // table reads go through the scalar unit (no vector-memory wait)
     scalar_load2(p.csr.ptr + lh * p.csr.ptr_sh + rb, p.csr.ptr + lh * p.csr.ptr_sh + rb + 1, e0, e1);
   }
   const int32_t *cols = p.csr.idx + lh * p.csr.idx_sh;
@@ -123,18 +146,56 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
   // Table entries: block e in col_cur (scalar register); block e + 1 is requested one block
   // early as a vector load (col_pending) and first used behind the next tile wait, so that no
   // table read ever stalls the loop.
-  int col_cur = e0 < e1 ? scalar_load(cols + e0) : 0;
-  int col_pending = e0 + 1 < e1 ? cols[e0 + 1] : 0;
-  if (e0 < e1) issue(col_cur, 0);
+  //
+  // RP: the workgroup walks the union of its two rows' entries in column order (both rows are
+  // sorted), merging them on the fly: head_a / head_b are the next unconsumed entries (scalar),
+  // pend_a / pend_b the entries after them (vector loads, consumed behind a tile wait like
+  // col_pending); flg says which rows hold the current column.  A wave pair whose row does not
+  // hold it only takes part in the copy and the barrier.
+  constexpr int kEnd = 0x7fffffff;
+  int col_cur = 0, col_pending = 0;
+  int a_pos = e0, b_pos = emid, head_a = kEnd, head_b = kEnd, pend_a = 0, pend_b = 0, flg_cur = 0;
+  if constexpr (RP) {
+    if (a_pos < emid) head_a = scalar_load(cols + a_pos);
+    if (b_pos < e1) head_b = scalar_load(cols + b_pos);
+    if (a_pos + 1 < emid) pend_a = cols[a_pos + 1];
+    if (b_pos + 1 < e1) pend_b = cols[b_pos + 1];
+    col_cur = min(head_a, head_b);
+    flg_cur = (head_a == col_cur ? 1 : 0) | (head_b == col_cur ? 2 : 0);
+    if (col_cur != kEnd) issue(col_cur, 0);
+  } else {
+    col_cur = e0 < e1 ? scalar_load(cols + e0) : 0;
+    col_pending = e0 + 1 < e1 ? cols[e0 + 1] : 0;
+    if (e0 < e1) issue(col_cur, 0);
+  }
   auto block_step = [&](int e, auto stage_tag) {
     constexpr int stage = decltype(stage_tag)::value;
     const int col = col_cur;
     wait_tile_loads();
     __syncthreads();  // tile e is visible; every wave is done with the other stage
-    const int col_next = __builtin_amdgcn_readfirstlane(col_pending);  // landed before the tile did
-    if (e + 2 < e1) col_pending = cols[e + 2];
-    if (e + 1 < e1) issue(col_next, stage ^ 1);
-    col_cur = col_next;
+    if constexpr (RP) {
+      const int flg = flg_cur;
+      if (flg & 1) {
+        ++a_pos;
+        head_a = a_pos < emid ? __builtin_amdgcn_readfirstlane(pend_a) : kEnd;
+        if (a_pos + 1 < emid) pend_a = cols[a_pos + 1];
+      }
+      if (flg & 2) {
+        ++b_pos;
+        head_b = b_pos < e1 ? __builtin_amdgcn_readfirstlane(pend_b) : kEnd;
+        if (b_pos + 1 < e1) pend_b = cols[b_pos + 1];
+      }
+      const int col_next = min(head_a, head_b);
+      flg_cur = (head_a == col_next ? 1 : 0) | (head_b == col_next ? 2 : 0);
+      if (col_next != kEnd) issue(col_next, stage ^ 1);
+      col_cur = col_next;
+      if (!((flg >> __builtin_amdgcn_readfirstlane(wave >> 1)) & 1)) return;  // not in this wave pair's row
+    } else {
+      const int col_next = __builtin_amdgcn_readfirstlane(col_pending);  // landed before the tile did
+      if (e + 2 < e1) col_pending = cols[e + 2];
+      if (e + 1 < e1) issue(col_next, stage ^ 1);
+      col_cur = col_next;
+    }
     const int key0 = col * 64;
     if (col < 0 || key0 >= sq.k_len || (p.causal && key0 > row0 + 31)) return;  // nothing visible (wave-uniform)
     constexpr int ks_ = stage * S::kStage, vs_ = ks_ + TL::kBytes;  // byte offsets of this stage's K and V tiles
@@ -228,9 +289,17 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
       for (int dt = 0; dt < DT; ++dt) oacc[dt] = M::mma(va[step & 1][dt], pb, oacc[dt]);
     }
   };
-  for (int e = e0; e < e1; e += 2) {
-    block_step(e, Const<0>{});
-    if (e + 1 < e1) block_step(e + 1, Const<1>{});
+  if constexpr (RP) {
+    while (col_cur != kEnd) {
+      block_step(0, Const<0>{});
+      if (col_cur == kEnd) break;
+      block_step(0, Const<1>{});
+    }
+  } else {
+    for (int e = e0; e < e1; e += 2) {
+      block_step(e, Const<0>{});
+      if (e + 1 < e1) block_step(e + 1, Const<1>{});
+    }
   }
 
   // l_run holds this lane's share of the row sum (keys with this lane's g)
@@ -519,9 +588,10 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
 // Explicit instantiations: with only the implicit ones the fp16 host stubs of
 // this kernel are not emitted by this compiler version.
 #define DK_INSTANTIATE_FWD(T, D, PAD)                                                  \
-  template __global__ void mfma_fwd_kernel<T, D, 1, PAD>(const FwdParams, int);       \
-  template __global__ void mfma_fwd_kernel<T, D, 2, PAD>(const FwdParams, int);       \
-  template __global__ void mfma_fwd_kernel<T, D, 4, PAD>(const FwdParams, int);       \
+  template __global__ void mfma_fwd_kernel<T, D, 1, PAD, false>(const FwdParams, int); \
+  template __global__ void mfma_fwd_kernel<T, D, 2, PAD, false>(const FwdParams, int); \
+  template __global__ void mfma_fwd_kernel<T, D, 2, PAD, true>(const FwdParams, int);  \
+  template __global__ void mfma_fwd_kernel<T, D, 4, PAD, false>(const FwdParams, int); \
   template __global__ void mfma_fwd_pipe_kernel<T, D, 1, PAD>(const FwdParams, int);
 DK_INSTANTIATE_FWD(bf16_t, 128, false)
 DK_INSTANTIATE_FWD(bf16_t, 64, false)
@@ -553,12 +623,7 @@ bool mfma_fwd_supported(const FwdParams &p, int dtype) {
 template <typename T, int D, int G, bool PAD>
 static int launch_tdg(const FwdParams &p, dim3 grid, int tiles_y, hipStream_t stream) {
   constexpr int smem = 2 * FwdSmem<D>::kStage;
-  static bool attr_set = false;  // raising the dynamic LDS limit is idempotent; a race only repeats it
-  if (!attr_set) {
-    DK_HIP_CHECK(hipFuncSetAttribute((const void *)mfma_fwd_kernel<T, D, G, PAD>,
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, smem));
-    attr_set = true;
-  }
+  DK_ALLOW_DYNAMIC_LDS((mfma_fwd_kernel<T, D, G, PAD, false>), smem);
   grid.x = p.Hq / G;
   // One head per workgroup (no head group to share tiles with) runs one wave per SIMD; there
   // the software-pipelined kernel is the faster one.  With two waves per SIMD it is not: it
@@ -566,23 +631,42 @@ static int launch_tdg(const FwdParams &p, dim3 grid, int tiles_y, hipStream_t st
   // between tile requests.  DKERNEL_FWD_PIPE=0 switches it off (A/B measurements).
   static const bool pipe = !(getenv("DKERNEL_FWD_PIPE") && atoi(getenv("DKERNEL_FWD_PIPE")) == 0);
   if constexpr (G == 1) if (pipe) {
-    static bool pipe_attr_set = false;
-    if (!pipe_attr_set) {
-      DK_HIP_CHECK(hipFuncSetAttribute((const void *)mfma_fwd_pipe_kernel<T, D, G, PAD>,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem));
-      pipe_attr_set = true;
-    }
+    DK_ALLOW_DYNAMIC_LDS((mfma_fwd_pipe_kernel<T, D, G, PAD>), smem);
     hipLaunchKernelGGL((mfma_fwd_pipe_kernel<T, D, G, PAD>), grid, dim3(128 * G), smem, stream, p, tiles_y);
     DK_HIP_CHECK(hipGetLastError());
     return DK_OK;
   }
-  hipLaunchKernelGGL((mfma_fwd_kernel<T, D, G, PAD>), grid, dim3(128 * G), smem, stream, p, tiles_y);
+  hipLaunchKernelGGL((mfma_fwd_kernel<T, D, G, PAD, false>), grid, dim3(128 * G), smem, stream, p, tiles_y);
+  DK_HIP_CHECK(hipGetLastError());
+  return DK_OK;
+}
+
+// One head per workgroup and every sequence in its own token dimension: two adjacent q tiles of
+// a head share a workgroup (and the K/V tiles their rows have in common), which gives the two
+// waves per SIMD that a single 64-row tile cannot.  DKERNEL_FWD_ROWPAIR=0 switches it off.
+template <typename T, int D, bool PAD>
+static int launch_row_pairs(const FwdParams &p, hipStream_t stream) {
+  const SeqView &s = p.seqs;
+  constexpr int smem = 2 * FwdSmem<D>::kStage;
+  DK_ALLOW_DYNAMIC_LDS((mfma_fwd_kernel<T, D, 2, PAD, true>), smem);
+  int pairs;
+  if (s.q_starts) {
+    pairs = (cdiv(s.max_q_len, 64) + 1) / 2 + 1;  // a sequence's rows start anywhere inside a pair
+  } else {
+    const int past = p.causal ? s.max_k_len - s.max_q_len : 0;
+    pairs = (((past + s.max_q_len - 1) / 64) >> 1) - ((past / 64) >> 1) + 1;
+  }
+  DK_REQUIRE(pairs <= 65535, "too many q tiles for one launch (%d)", pairs);
+  hipLaunchKernelGGL((mfma_fwd_kernel<T, D, 2, PAD, true>), dim3(p.Hq, pairs, s.batch), dim3(256), smem, stream, p,
+                     pairs);
   DK_HIP_CHECK(hipGetLastError());
   return DK_OK;
 }
 
 template <typename T, int D, bool PAD>
 static int launch_tdp(const FwdParams &p, dim3 grid, int tiles_y, hipStream_t stream) {
+  static const bool row_pairs = !(getenv("DKERNEL_FWD_ROWPAIR") && atoi(getenv("DKERNEL_FWD_ROWPAIR")) == 0);
+  if (row_pairs && !p.seqs.packed && fwd_group(p) == 1) return launch_row_pairs<T, D, PAD>(p, stream);
   switch (fwd_group(p)) {
     case 4: return launch_tdg<T, D, 4, PAD>(p, grid, tiles_y, stream);
     case 2: return launch_tdg<T, D, 2, PAD>(p, grid, tiles_y, stream);

@@ -375,6 +375,49 @@ def test_c4_user_pattern_varlen_partitions(impl):
         s += l
 
 
+@pytest.mark.parametrize("D,dtype", [(128, torch.bfloat16), (64, torch.float16), (96, torch.bfloat16)])
+def test_row_pairs_user_pattern_and_offsets(D, dtype):
+    """One head per workgroup and unpacked inputs: two adjacent q tiles share a workgroup and
+    merge their table rows on the fly.  A random per-head pattern (rows that share few columns,
+    rows with one entry, empty partitions), odd numbers of row blocks, k longer than q (the first
+    row block is the odd half of a pair) and left / right padding exercise that merge."""
+    H, bs, nb = 3, 64, 24
+    sm = 1 / math.sqrt(D)
+    g = torch.Generator().manual_seed(7)
+    pat = (torch.rand(H, nb, nb, generator=g) < 0.25)
+    pat |= torch.eye(nb, dtype=torch.bool)[None]
+    pat[:, 5, :5] = False            # a row with its diagonal block only
+    pat = torch.tril(pat.to(torch.uint8))
+    import warnings
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        mod = SparseAttention(bs, pat).to(DEV)
+    bm = pat.numpy()
+    for Lq, Lk in ((nb * 64, nb * 64), (700, 700), (64, 64), (65, 65), (300, 1000), (1, 129), (200, 264)):
+        print(f"row pairs: D={D} Lq={Lq} Lk={Lk}", flush=True)
+        q = torch.randn(2, Lq, H, D, generator=g).to(dtype)
+        k, v = (torch.randn(2, Lk, H, D, generator=g).to(dtype) for _ in range(2))
+        out, lse = mod(q.to(DEV), k.to(DEV), v.to(DEV), sm, return_lse=True)
+        for b in range(2):
+            ro, rl = _seq_oracle(q[b], k[b], v[b], bm, bs, sm)
+            assert_close(f"O[{b}]", out[b], ro, **TOL)
+            assert_close(f"LSE[{b}]", lse[b], rl.transpose(0, 1) if rl.shape != lse[b].shape else rl, atol=LSE_TOL, rtol=0)
+    # left-padded and right-padded prefill (per-sequence offsets, unpacked)
+    Lmax, lens = 1024, [1024, 1, 333, 640]
+    q, k, v = (torch.randn(len(lens), Lmax, H, D, generator=g).to(dtype) for _ in range(3))
+    for left in (True, False):
+        qp, kp, vp = torch.zeros_like(q), torch.zeros_like(k), torch.zeros_like(v)
+        for i, l in enumerate(lens):
+            sl = slice(Lmax - l, Lmax) if left else slice(0, l)
+            qp[i, sl], kp[i, sl], vp[i, sl] = q[i, :l], k[i, :l], v[i, :l]
+        extra = dict(left_paddings=torch.tensor([Lmax - l for l in lens])) if left else dict(seqlens=torch.tensor(lens))
+        out = mod(qp.to(DEV), kp.to(DEV), vp.to(DEV), sm, **extra)
+        for i, l in enumerate(lens):
+            sl = slice(Lmax - l, Lmax) if left else slice(0, l)
+            ro, _ = _seq_oracle(q[i, :l], k[i, :l], v[i, :l], bm, bs, sm)
+            assert_close(f"O padded[{i}] left={left}", out[i, sl], ro, **TOL)
+
+
 def test_seq_partition_with_backward(impl):
     """Context-parallel emulation in one process (reference:
     tests/test_seq_partition.py): q chunks x kv partitions, non-square masks,

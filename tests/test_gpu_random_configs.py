@@ -1,0 +1,188 @@
+"""GPU differential test over seeded random configurations: the matrix-core
+kernels ("auto") against the independent generic fp32 kernels on the same
+inputs, and both against the fp32 dense oracle where the case is small enough.
+The draw covers what selects a kernel variant: heads per kv head (group of 4,
+2, 1 -> head groups, row pairs), head dims (multiples of 8 up to 128 ->
+zero-padded tiles), pattern blocks (64 / 128 / 256 -> split tables), lengths
+that are not multiples of the block, k longer than q, local / vertical
+parameters, dense heads, bf16 / fp16, token or head major layout, forward and
+backward with and without a gradient through LSE."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from dkernel_amd import LocalStrideSparseAttention, ops
+from oracle import layout as OL
+from helpers import LSE_TOL, TOL, assert_close, expand_heads, oracle_fwd
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def draw_config(rng):
+    ratio = int(rng.choice([1, 1, 2, 4, 8]))
+    Hkv = int(rng.choice([1, 2, 3]))
+    Hq = Hkv * ratio
+    bs = int(rng.choice([64, 64, 64, 128, 256]))
+    D = int(rng.choice([128, 128, 64, 96, 48, 80, 112, 32]))
+    nb = int(rng.integers(1, 13)) if bs == 64 else int(rng.integers(1, 6))
+    L = int(rng.integers((nb - 1) * bs + 1, nb * bs + 1))
+    past = int(rng.choice([0, 0, 0, 64, 37, 200])) if L > 1 else 0
+    local = int(rng.integers(1, 5))
+    vert = int(rng.integers(1, 7))
+    dense = int(rng.integers(0, 2)) if Hkv > 1 else 0
+    dtype = torch.bfloat16 if rng.random() < 0.7 else torch.float16
+    seq_dim = int(rng.choice([1, 1, 2]))
+    B = int(rng.integers(1, 4))
+    return dict(B=B, Hq=Hq, Hkv=Hkv, bs=bs, D=D, Lq=L, Lk=L + past, local=local, vert=vert, dense=dense,
+                dtype=dtype, seq_dim=seq_dim, dlse=bool(rng.random() < 0.3), backward=past == 0)
+
+
+def run_impl(impl, mod, q, k, v, do, dlse, sm, backward):
+    ops.set_impl(impl)
+    try:
+        qd, kd, vd = (x.to(DEV).requires_grad_(backward) for x in (q, k, v))
+        out, lse = mod(qd, kd, vd, sm, return_lse=True)
+        res = [out.detach().cpu(), lse.detach().cpu()]
+        if backward:
+            loss = (out.float() * do.to(DEV).float()).sum()
+            if dlse is not None:
+                loss = loss + (lse * dlse.to(DEV)).sum()
+            loss.backward()
+            res += [qd.grad.cpu(), kd.grad.cpu(), vd.grad.cpu()]
+        return res
+    finally:
+        ops.set_impl("auto")
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_config_matches_generic_kernels_and_oracle(seed):
+    rng = np.random.default_rng(1000 + seed)
+    c = draw_config(rng)
+    print("config", {k: str(v) for k, v in c.items()}, flush=True)
+    g = torch.Generator().manual_seed(seed)
+    B, Hq, Hkv, D, Lq, Lk, sd = c["B"], c["Hq"], c["Hkv"], c["D"], c["Lq"], c["Lk"], c["seq_dim"]
+
+    def draw(L, H):
+        shape = (B, L, H, D) if sd == 1 else (B, H, L, D)
+        return torch.randn(shape, generator=g, dtype=torch.float32).to(c["dtype"])
+    q, k, v, do = draw(Lq, Hq), draw(Lk, Hkv), draw(Lk, Hkv), draw(Lq, Hq)
+    dlse = torch.randn(B, Hq, Lq, generator=g) if (c["dlse"] and c["backward"]) else None
+    sm = 1.0 / math.sqrt(D)
+    kw = dict(seq_dim=sd)
+    if Hkv != Hq:
+        kw["num_kv_heads"] = Hkv
+    if c["dense"]:
+        kw["num_dense_heads"] = c["dense"]
+    max_len = ((Lk + max(c["bs"], 64) - 1) // max(c["bs"], 64)) * max(c["bs"], 64)
+    mod = LocalStrideSparseAttention(Hq, max_len, c["bs"], c["local"], c["vert"], **kw).to(DEV)
+    got = run_impl("auto", mod, q, k, v, do, dlse, sm, c["backward"])
+    ref = run_impl("generic", mod, q, k, v, do, dlse, sm, c["backward"])
+    names = ["O", "LSE", "dQ", "dK", "dV"]
+    for name, a, b in zip(names, got, ref):
+        if name == "LSE":
+            assert_close(f"{name} auto vs generic", a, b, atol=LSE_TOL, rtol=0)
+        else:
+            assert_close(f"{name} auto vs generic", a, b, **TOL)
+    # oracle on the same inputs (dense fp32 attention with the token mask of the block pattern)
+    mkw = {k_: v_ for k_, v_ in kw.items() if k_ in ("num_kv_heads", "num_dense_heads")}
+    bm = expand_heads(OL.block_mask(Hq, max_len, c["bs"], c["local"], c["vert"], **mkw), Hq)
+    qo, ko, vo = (x.float().requires_grad_(c["backward"]) for x in (q, k, v))
+    ro, rl = oracle_fwd(qo, ko, vo, bm, c["bs"], sm, seq_dim=sd)
+    assert_close("O vs oracle", got[0], ro, **TOL)
+    assert_close("LSE vs oracle", got[1], rl, atol=LSE_TOL, rtol=0)
+    if c["backward"]:
+        loss = (ro * do.float()).sum()
+        if dlse is not None:
+            loss = loss + (rl * dlse).sum()
+        loss.backward()
+        for name, a, b in zip(names[2:], got[2:], (qo.grad, ko.grad, vo.grad)):
+            assert_close(f"{name} vs oracle", a, b, **TOL)
+
+
+def _seq_oracle(q, k, v, bm, bs, sm):
+    """One sequence, (L, H, D) tensors; the queries are the last positions of the keys."""
+    from oracle import attention as OA
+    mask = OA.sequence_token_mask(bm, bs, q.shape[0], k.shape[0], causal=True)
+    o, lse = OA.dense_attention(q[None], k[None], v[None], torch.from_numpy(mask), sm, seq_dim=1)
+    return o[0], lse[0]
+
+
+@pytest.mark.parametrize("seed", range(30))
+def test_random_inference_config_matches_generic_kernels_and_oracle(seed):
+    """Per-sequence lengths: left-padded, right-padded and packed prefill, padded and packed
+    single-token decode (split-KV kernels), chunked packed prefill."""
+    rng = np.random.default_rng(5000 + seed)
+    ratio = int(rng.choice([1, 2, 4]))
+    Hkv = int(rng.choice([1, 2]))
+    Hq = Hkv * ratio
+    bs = int(rng.choice([64, 64, 128]))
+    D = int(rng.choice([128, 64, 96, 40]))
+    dtype = torch.bfloat16 if rng.random() < 0.7 else torch.float16
+    mode = str(rng.choice(["left", "right", "packed", "packed_decode", "left_decode", "right_decode", "chunked"]))
+    nseq = int(rng.integers(1, 6))
+    Lmax = int(rng.choice([256, 512, 1024]))
+    lens = [int(rng.integers(1, Lmax + 1)) for _ in range(nseq)]
+    local, vert = int(rng.integers(1, 4)), int(rng.integers(1, 6))
+    print("config", dict(Hq=Hq, Hkv=Hkv, bs=bs, D=D, dtype=str(dtype), mode=mode, lens=lens, local=local, vert=vert),
+          flush=True)
+    sm = 1.0 / math.sqrt(D)
+    g = torch.Generator().manual_seed(seed)
+    kw = dict(num_kv_heads=Hkv) if Hkv != Hq else {}
+    mod = LocalStrideSparseAttention(Hq, Lmax, bs, local, vert, **kw).to(DEV)
+    bm = expand_heads(OL.block_mask(Hq, Lmax, bs, local, vert, **kw), Hq)
+    ks = [torch.randn(l, Hkv, D, generator=g).to(dtype) for l in lens]
+    vs = [torch.randn(l, Hkv, D, generator=g).to(dtype) for l in lens]
+    decode = mode.endswith("decode")
+    if mode == "chunked":
+        qlens = [int(rng.integers(1, l + 1)) for l in lens]
+    else:
+        qlens = [1 if decode else l for l in lens]
+    qs = [torch.randn(ql, Hq, D, generator=g).to(dtype) for ql in qlens]
+
+    def call():
+        if mode in ("packed", "packed_decode", "chunked"):
+            cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32).to(DEV)
+            extra = dict(cu_seqlen_k=cu)
+            if mode == "chunked":
+                extra["cu_seqlen_q"] = torch.tensor([0] + list(np.cumsum(qlens)), dtype=torch.int32).to(DEV)
+            out, lse = mod(torch.cat(qs).to(DEV), torch.cat(ks).to(DEV), torch.cat(vs).to(DEV), sm,
+                           return_lse=True, **extra)
+            out, lse = out.cpu(), lse.cpu()
+            offs = np.cumsum([0] + qlens)
+            return [(out[offs[i]:offs[i + 1]], lse[:, offs[i]:offs[i + 1]]) for i in range(nseq)]
+        left = mode.startswith("left")
+        Lq = 1 if decode else Lmax
+        qp = torch.zeros(nseq, Lq, Hq, D, dtype=dtype)
+        kp, vp = torch.zeros(nseq, Lmax, Hkv, D, dtype=dtype), torch.zeros(nseq, Lmax, Hkv, D, dtype=dtype)
+        for i, l in enumerate(lens):
+            sl = slice(Lmax - l, Lmax) if left else slice(0, l)
+            kp[i, sl], vp[i, sl] = ks[i], vs[i]
+            if decode:
+                qp[i] = qs[i]
+            else:
+                qp[i, sl] = qs[i]
+        extra = dict(left_paddings=torch.tensor([Lmax - l for l in lens])) if left else dict(seqlens=torch.tensor(lens))
+        out, lse = mod(qp.to(DEV), kp.to(DEV), vp.to(DEV), sm, return_lse=True, **extra)
+        out, lse = out.cpu(), lse.cpu()
+        res = []
+        for i, l in enumerate(lens):
+            sl = slice(0, 1) if decode else (slice(Lmax - l, Lmax) if left else slice(0, l))
+            res.append((out[i, sl], lse[i][:, sl]))
+        return res
+
+    def with_impl(name):
+        ops.set_impl(name)
+        try:
+            return call()
+        finally:
+            ops.set_impl("auto")
+    got, ref = with_impl("auto"), with_impl("generic")
+    for i in range(nseq):
+        assert_close(f"O[{i}] auto vs generic", got[i][0], ref[i][0], **TOL)
+        assert_close(f"LSE[{i}] auto vs generic", got[i][1], ref[i][1], atol=LSE_TOL, rtol=0)
+        ro, rl = _seq_oracle(qs[i], ks[i], vs[i], bm, bs, sm)
+        assert_close(f"O[{i}] vs oracle", got[i][0], ro, **TOL)
+        assert_close(f"LSE[{i}] vs oracle", got[i][1], rl, atol=LSE_TOL, rtol=0)

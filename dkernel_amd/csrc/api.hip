@@ -27,7 +27,7 @@ static RowView view(const dk_rowvec &t) { return RowView{t.ptr, t.stride_b, t.st
 static LutView view(const dk_lut &l) {
   return LutView{l.ptr, l.idx, l.ptr_stride_h, l.idx_stride_h, l.entry_width, l.num_heads,
                  l.num_rows, l.block_rows, l.block_cols, l.group < 1 ? 1 : l.group,
-                 l.max_row_entries};
+                 l.max_row_entries, l.sub_block};
 }
 static SeqView view(const dk_seqs &s) {
   return SeqView{s.batch, s.max_q_len, s.max_k_len, s.packed, s.q_starts, s.q_ends, s.k_starts, s.k_ends};
@@ -48,6 +48,9 @@ static int check_lut(const dk_lut &l, const char *name, int Hq, int Hkv) {
              "%s tile sizes must be powers of 2 in [16, 1024], got (%d, %d)", name, l.block_rows, l.block_cols);
   DK_REQUIRE(l.entry_width == 1 || l.entry_width == 2, "%s entry_width must be 1 or 2", name);
   DK_REQUIRE(l.num_rows >= 0, "%s num_rows negative", name);
+  DK_REQUIRE(l.sub_block == 0 || ((l.sub_block == 16 || l.sub_block == 32) && l.entry_width == 2 &&
+                                  l.block_rows == 64 && l.block_cols == 64),
+             "%s sub_block must be 0, or 16 / 32 with entry_width 2 and 64 x 64 tiles", name);
   return DK_OK;
 }
 
@@ -174,6 +177,9 @@ int dk_fwd(const dk_fwd_args *a) {
       return fail(DK_ERR_UNSUPPORTED, "no MFMA forward kernel for dtype %d, head_dim %d, tiles (%d, %d)", a->dtype,
                   p.D, p.csr.block_rows, p.csr.block_cols);
   }
+  if (p.csr.sub_block)
+    return fail(DK_ERR_UNSUPPORTED, "tables with sub-block masks need the matrix-core kernels (dtype %d, head_dim %d)",
+                a->dtype, p.D);
   return launch_generic_fwd(p, a->dtype, stream);
 }
 
@@ -200,6 +206,9 @@ int dk_bwd(const dk_bwd_args *a) {
       return fail(DK_ERR_UNSUPPORTED, "no MFMA backward kernel for dtype %d, head_dim %d, tiles (%d, %d)",
                   a->dtype, p.D, p.csr.block_rows, p.csr.block_cols);
   }
+  if (p.csr.sub_block || p.csc.sub_block)
+    return fail(DK_ERR_UNSUPPORTED, "tables with sub-block masks need the matrix-core kernels (dtype %d, head_dim %d)",
+                a->dtype, p.D);
   return launch_generic_bwd(p, a->dtype, stream);
 }
 

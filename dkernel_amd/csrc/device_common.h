@@ -50,7 +50,7 @@ struct RowView {
 struct LutView {
   const int32_t *ptr, *idx;
   int64_t ptr_sh, idx_sh;
-  int32_t entry_width, num_heads, num_rows, block_rows, block_cols, group, max_row_entries;
+  int32_t entry_width, num_heads, num_rows, block_rows, block_cols, group, max_row_entries, sub_block;
 };
 struct SeqView {
   int32_t batch, max_q_len, max_k_len, packed;

@@ -37,7 +37,7 @@ struct FwdSmem {  // one stage = K tile + V tile, swizzled row-major (mfma_commo
   static constexpr int kStage = 2 * Tile<D>::kBytes;
 };
 
-template <typename T, int D, int G, bool PAD, bool RP>
+template <typename T, int D, int G, bool PAD, bool RP, bool SUB = false>
 __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 ? 1 : 2, 2))) void mfma_fwd_kernel(const FwdParams p, int tiles_y) {
   using M = Mma<T>;
   using vec8 = typename M::vec8;
@@ -49,6 +49,9 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
   extern __shared__ __align__(16) char smem[];
 
   static_assert(!RP || G == 2, "row pairs: two wave pairs, one q tile each");
+  // SUB: table entries are (column, bit mask over the pattern blocks inside the 64 x 64 tile)
+  static_assert(!SUB || (!RP && !PAD), "sub-block masks: plain tiles only");
+  constexpr int EW = SUB ? 2 : 1;  // ints per table entry
   SeqInfo sq;
   int tile;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -154,6 +157,7 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
   // hold it only takes part in the copy and the barrier.
   constexpr int kEnd = 0x7fffffff;
   int col_cur = 0, col_pending = 0;
+  int bits_cur = 0, bits_pending = 0;  // SUB: the entry's mask, carried like the column
   int a_pos = e0, b_pos = emid, head_a = kEnd, head_b = kEnd, pend_a = 0, pend_b = 0, flg_cur = 0;
   if constexpr (RP) {
     if (a_pos < emid) head_a = scalar_load(cols + a_pos);
@@ -164,13 +168,18 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
     flg_cur = (head_a == col_cur ? 1 : 0) | (head_b == col_cur ? 2 : 0);
     if (col_cur != kEnd) issue(col_cur, 0);
   } else {
-    col_cur = e0 < e1 ? scalar_load(cols + e0) : 0;
-    col_pending = e0 + 1 < e1 ? cols[e0 + 1] : 0;
+    col_cur = e0 < e1 ? scalar_load(cols + e0 * EW) : 0;
+    col_pending = e0 + 1 < e1 ? cols[(e0 + 1) * EW] : 0;
+    if constexpr (SUB) {
+      bits_cur = e0 < e1 ? scalar_load(cols + e0 * EW + 1) : 0;
+      bits_pending = e0 + 1 < e1 ? cols[(e0 + 1) * EW + 1] : 0;
+    }
     if (e0 < e1) issue(col_cur, 0);
   }
   auto block_step = [&](int e, auto stage_tag) {
     constexpr int stage = decltype(stage_tag)::value;
     const int col = col_cur;
+    const int bits = bits_cur;
     wait_tile_loads();
     __syncthreads();  // tile e is visible; every wave is done with the other stage
     if constexpr (RP) {
@@ -192,7 +201,11 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
       if (!((flg >> __builtin_amdgcn_readfirstlane(wave >> 1)) & 1)) return;  // not in this wave pair's row
     } else {
       const int col_next = __builtin_amdgcn_readfirstlane(col_pending);  // landed before the tile did
-      if (e + 2 < e1) col_pending = cols[e + 2];
+      if constexpr (SUB) bits_cur = __builtin_amdgcn_readfirstlane(bits_pending);
+      if (e + 2 < e1) {
+        col_pending = cols[(e + 2) * EW];
+        if constexpr (SUB) bits_pending = cols[(e + 2) * EW + 1];
+      }
       if (e + 1 < e1) issue(col_next, stage ^ 1);
       col_cur = col_next;
     }
@@ -233,6 +246,23 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
     // 32nt + 8(r/4) + 4g + r%4.  m_run is a reference maximum that is only
     // raised when a row's maximum grows by more than 2^8 (the accumulator
     // and the row sum stay consistent with it, so the result is exact).
+    if constexpr (SUB) {
+      // pattern blocks of the tile that this row does not attend: bit (row part) * f + (key part)
+      const int lb = p.csr.sub_block == 16 ? 4 : 5, f = 64 >> lb;
+      const int full = f == 4 ? 0xffff : 0xf;
+      if ((bits & full) != full) {  // wave-uniform
+        const int row_part = ((wave & 1) * 32 + m) >> lb;
+        const int row_bits = bits >> (row_part * f);
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            // key 32 nt + 8 (r / 4) + 4 g + r % 4: the last two terms stay inside a part of >= 16 keys
+            const int key_part = (nt * 32 + (r >> 2) * 8) >> lb;
+            sacc[nt][r] = ((row_bits >> key_part) & 1) ? sacc[nt][r] : -INFINITY;
+          }
+      }
+    }
     const bool need_mask = (key0 + 63 >= sq.k_len) || (p.causal && key0 + 63 > row0);
     if (need_mask) {
       const int lim = p.causal ? min(pos, sq.k_len - 1) : sq.k_len - 1;  // last visible key of this row
@@ -593,6 +623,15 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
   template __global__ void mfma_fwd_kernel<T, D, 2, PAD, true>(const FwdParams, int);  \
   template __global__ void mfma_fwd_kernel<T, D, 4, PAD, false>(const FwdParams, int); \
   template __global__ void mfma_fwd_pipe_kernel<T, D, 1, PAD>(const FwdParams, int);
+#define DK_INSTANTIATE_FWD_SUB(T, D)                                                                  \
+  template __global__ void mfma_fwd_kernel<T, D, 1, false, false, true>(const FwdParams, int); \
+  template __global__ void mfma_fwd_kernel<T, D, 2, false, false, true>(const FwdParams, int); \
+  template __global__ void mfma_fwd_kernel<T, D, 4, false, false, true>(const FwdParams, int);
+DK_INSTANTIATE_FWD_SUB(bf16_t, 128)
+DK_INSTANTIATE_FWD_SUB(bf16_t, 64)
+DK_INSTANTIATE_FWD_SUB(f16_t, 128)
+DK_INSTANTIATE_FWD_SUB(f16_t, 64)
+#undef DK_INSTANTIATE_FWD_SUB
 DK_INSTANTIATE_FWD(bf16_t, 128, false)
 DK_INSTANTIATE_FWD(bf16_t, 64, false)
 DK_INSTANTIATE_FWD(f16_t, 128, false)
@@ -617,7 +656,8 @@ static int fwd_group(const FwdParams &p) {
 
 bool mfma_fwd_supported(const FwdParams &p, int dtype) {
   return (dtype == DK_BF16 || dtype == DK_F16) && mfma_head_dim_ok(p.D) && p.csr.block_rows == 64 &&
-         p.csr.block_cols == 64 && p.csr.entry_width == 1 && p.vec_ok;
+         p.csr.block_cols == 64 && p.vec_ok &&
+         (p.csr.entry_width == 1 || (p.csr.sub_block != 0 && (p.D == 64 || p.D == 128)));
 }
 
 template <typename T, int D, int G, bool PAD>
@@ -674,9 +714,33 @@ static int launch_tdp(const FwdParams &p, dim3 grid, int tiles_y, hipStream_t st
   }
 }
 
+// Tables whose entries carry a bit mask over the pattern's 16- or 32-token blocks inside each
+// 64 x 64 tile: the plain kernel with the mask applied to S (no row pairs, no padded head dims).
+template <typename T, int D, int G>
+static int launch_sub_g(const FwdParams &p, dim3 grid, int tiles_y, hipStream_t stream) {
+  constexpr int smem = 2 * FwdSmem<D>::kStage;
+  DK_ALLOW_DYNAMIC_LDS((mfma_fwd_kernel<T, D, G, false, false, true>), smem);
+  grid.x = p.Hq / G;
+  hipLaunchKernelGGL((mfma_fwd_kernel<T, D, G, false, false, true>), grid, dim3(128 * G), smem, stream, p, tiles_y);
+  DK_HIP_CHECK(hipGetLastError());
+  return DK_OK;
+}
+
+template <typename T, int D>
+static int launch_sub(const FwdParams &p, dim3 grid, int tiles_y, hipStream_t stream) {
+  switch (fwd_group(p)) {
+    case 4: return launch_sub_g<T, D, 4>(p, grid, tiles_y, stream);
+    case 2: return launch_sub_g<T, D, 2>(p, grid, tiles_y, stream);
+    default: return launch_sub_g<T, D, 1>(p, grid, tiles_y, stream);
+  }
+}
+
 // head dims below the tile width (64 or 128) run the zero-padded instantiation
 template <typename T>
 static int launch_t(const FwdParams &p, dim3 grid, int tiles_y, hipStream_t stream) {
+  if (p.csr.sub_block) {
+    return p.D == 128 ? launch_sub<T, 128>(p, grid, tiles_y, stream) : launch_sub<T, 64>(p, grid, tiles_y, stream);
+  }
   if (p.D == 128) return launch_tdp<T, 128, false>(p, grid, tiles_y, stream);
   if (p.D == 64) return launch_tdp<T, 64, false>(p, grid, tiles_y, stream);
   return p.D > 64 ? launch_tdp<T, 128, true>(p, grid, tiles_y, stream) : launch_tdp<T, 64, true>(p, grid, tiles_y, stream);

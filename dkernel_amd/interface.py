@@ -16,8 +16,8 @@ from torch import Tensor
 
 from .ops import _sparse_attention
 from .utils import (dense_to_ccol_row, get_sparse_attn_mask, is_kv_cache_efficient,
-                    merge_split_fwd_kernel_blocks, multiple_of, split_tile_tables, verify_sparse_pattern,
-                    zero_stride)
+                    masked_tile_tables, merge_split_fwd_kernel_blocks, multiple_of, split_tile_tables,
+                    verify_sparse_pattern, zero_stride)
 
 _KERNEL_TILE = 64  # q and k tile of the matrix-core kernels
 
@@ -80,6 +80,9 @@ class SparseAttention(torch.nn.Module):
         # Patterns with blocks larger than the 64 x 64 tile of the matrix-core kernels run on
         # tables split to that tile, unless the caller fixes the tile sizes.
         split_for_kernels = block_m is None and block_n is None and block_size > _KERNEL_TILE
+        # ... and patterns with smaller blocks on tile tables whose entries carry a bit mask over
+        # the pattern blocks inside the tile (forward only; backward keeps the tables above)
+        mask_for_kernels = block_m is None and block_n is None and block_size < _KERNEL_TILE
         if block_m is None:
             block_m = max(block_size, 64) if causal else block_size
         if block_n is None:
@@ -151,6 +154,18 @@ class SparseAttention(torch.nn.Module):
             self.register_buffer("kernel_csc_ccol", tile_csc[0].to(torch.int32), persistent=False)
             self.register_buffer("kernel_csc_row", tile_csc[1].to(torch.int32), persistent=False)
 
+        self.mask_tile = None
+        if mask_for_kernels:
+            m_csr, _ = masked_tile_tables(block_size, sparse_pattern, _KERNEL_TILE)
+            m_csr = list(m_csr)
+            if m_csr[0].size(0) == 1:
+                m_csr = [zero_stride(x) for x in m_csr]
+            crow = m_csr[0]
+            self.mask_tile = _KERNEL_TILE
+            self.mask_lut_max_row = int((crow[:, 1:] - crow[:, :-1]).max()) if crow.size(1) > 1 else 0
+            self.register_buffer("masked_csr_crow", m_csr[0].to(torch.int32), persistent=False)
+            self.register_buffer("masked_csr_col", m_csr[1].to(torch.int32), persistent=False)
+
     def forward(self,
                 q: Tensor,
                 k: Optional[Tensor] = None,
@@ -188,6 +203,10 @@ class SparseAttention(torch.nn.Module):
         else:
             layout_csr = (self.layout_csr_crow, self.layout_csr_col, self.block_m, self.block_n)
             layout_csc = (self.layout_csc_ccol, self.layout_csc_row, self.block_m2, self.block_n2)
+        if self.mask_tile is not None:
+            # (crow, (col, mask), tile rows, tile cols, pattern block size), longest row
+            kwargs["masked_fwd_layout"] = ((self.masked_csr_crow, self.masked_csr_col, self.mask_tile,
+                                            self.mask_tile, self.block_size), self.mask_lut_max_row)
         output, lse = _sparse_attention.apply(
             q, k, v, sm_scale, layout_csr, layout_csc,
             self.seq_dim, inf_kwargs, kwargs)

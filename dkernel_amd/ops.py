@@ -35,6 +35,20 @@ def set_impl(name: str) -> None:
     _impl = _IMPL[name]
 
 
+def _matrix_core_forward_applies(q: Tensor, k: Tensor, v: Tensor, out: Optional[Tensor]) -> bool:
+    """Whether dk_fwd will run these inputs on the matrix-core kernels with a masked tile table:
+    16-bit floats, head_dim 64 or 128, 16-byte aligned rows (the library's own conditions; it
+    fails loudly if they were judged wrong here)."""
+    if _impl == _lib.DK_IMPL_GENERIC or q.dtype not in (torch.bfloat16, torch.float16):
+        return False
+    if q.size(-1) not in (64, 128):
+        return False
+    for x in (q, k, v) + ((out,) if out is not None else ()):
+        if x.stride(-1) != 1 or x.data_ptr() % 16 or any(st % 8 for st in x.stride()[:-1]):
+            return False
+    return True
+
+
 def _require_gpu(*xs: Tensor) -> None:
     for x in xs:
         if not x.is_cuda:
@@ -66,7 +80,8 @@ def _rowvec(x: Optional[Tensor], strides=None) -> _lib.RowVec:
 
 
 def _lut(layout: Tuple[Tensor, Tensor, int, int], device, group: int = 1, max_row: int = 0) -> _lib.Lut:
-    ptr, idx, block_rows, block_cols = layout
+    ptr, idx, block_rows, block_cols = layout[:4]
+    sub_block = int(layout[4]) if len(layout) > 4 else 0  # entries carry a bit mask over pattern blocks
     assert ptr.dtype == torch.int32 and idx.dtype == torch.int32
     assert ptr.device == device and idx.device == device, \
         "sparse layout is on another device than q; move the module with .to(device)"
@@ -80,7 +95,8 @@ def _lut(layout: Tuple[Tensor, Tensor, int, int], device, group: int = 1, max_ro
     else:
         assert idx.stride(-1) == 1 or idx.size(-1) <= 1
     return _lib.Lut(ptr.data_ptr(), idx.data_ptr(), ptr.stride(0), idx.stride(0), width,
-                    ptr.size(0), ptr.size(1) - 1, int(block_rows), int(block_cols), int(group), int(max_row))
+                    ptr.size(0), ptr.size(1) - 1, int(block_rows), int(block_cols), int(group), int(max_row),
+                    sub_block)
 
 
 _CONST_I32 = {}
@@ -396,6 +412,14 @@ class _sparse_attention(torch.autograd.Function):
              f"but the number of heads in the sparse pattern is {layout_csr_crow.size(0)}")
         sm_scale = sm_scale or 1. / math.sqrt(float(q.size(-1)))
 
+        # Patterns with blocks below the kernel tile: the forward runs on the masked tile table
+        # whenever the matrix-core kernels take these inputs; backward keeps the module's tables.
+        masked = kwargs.get("masked_fwd_layout", None)
+        if masked is not None and _matrix_core_forward_applies(q, k, v, kwargs.get("out", None)):
+            layout_csr, lut_max_row = masked
+        else:
+            lut_max_row = kwargs.get("lut_max_row", 0)
+
         if q.dim() == 3:
             assert inf_kwargs.get("cu_seqlen_k", None) is not None
             ctx.support_backward = False
@@ -416,14 +440,15 @@ class _sparse_attention(torch.autograd.Function):
                 res = padded_sparse_attn(q, k, v, sm_scale, layout_csr, left_paddings=left_paddings,
                                          seqlens=seqlens, seq_dim=seq_dim, max_seqlen=max_seqlen,
                                          causal=causal, return_lse=return_lse, lut_group=lut_group,
-                                         lut_max_row=kwargs.get("lut_max_row", 0))
+                                         lut_max_row=lut_max_row)
                 output, lse = res if return_lse else (res, None)
             else:
                 ctx.support_backward = True
                 ctx.message = ""
                 fwd_kwargs = {k_: v_ for k_, v_ in kwargs.items()
                               if k_ in ("inference", "out", "d_splits", "max_seqlen", "return_lse",
-                                        "causal", "split_qkv", "lut_group", "lut_max_row")}
+                                        "causal", "split_qkv", "lut_group")}
+                fwd_kwargs["lut_max_row"] = lut_max_row
                 output, lse = _forward(ctx, q, k, v, sm_scale, layout_csr, seq_dim=seq_dim, **fwd_kwargs)
         return output, lse
 

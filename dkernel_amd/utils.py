@@ -241,6 +241,28 @@ def split_tile_tables(block_size: int, sparse_pattern: Tensor, tile: int,
     return dense_to_crow_col(out), dense_to_ccol_row(out)
 
 
+def masked_tile_tables(block_size: int, sparse_pattern: Tensor, tile: int
+                       ) -> Tuple[Tuple[Tensor, Tensor], Tuple[Tensor, Tensor]]:
+    """CSR and CSC tables of a pattern whose blocks are smaller than the kernel
+    tile: one entry per tile x tile tile that holds any active block, with a
+    bit mask over the f x f pattern blocks inside it on the trailing dim
+    (bit i * f + j: row part i, column part j; f = tile // block_size).  The
+    pattern is zero-padded to whole tiles.  The reference has no counterpart
+    (its kernels take tiles of the block size)."""
+    assert tile % block_size == 0 and tile > block_size
+    f = tile // block_size
+    assert f * f <= 16
+    p = (sparse_pattern != 0).to("cpu", torch.int32)
+    H, M, N = p.shape
+    Mp, Np = cdiv(M, f) * f, cdiv(N, f) * f
+    padded = torch.zeros((H, Mp, Np), dtype=torch.int32)
+    padded[:, :M, :N] = p
+    weight = (1 << (torch.arange(f)[:, None] * f + torch.arange(f)[None, :])).to(torch.int32)
+    bits = (padded.view(H, Mp // f, f, Np // f, f) * weight[None, None, :, None, :]).sum(dim=(2, 4)).to(torch.int32)
+    bits = bits.to(sparse_pattern.device)
+    return dense_to_crow_col(bits, include_values=True), dense_to_ccol_row(bits, include_values=True)
+
+
 def zero_stride(x: Tensor, dim=0) -> Tensor:
     """Stride 0 on a broadcastable dim of size <= 1.  Reference: dkernel/utils.py:313-320."""
     assert x.size(dim) <= 1, f"Cannot set stride at {dim=} to 0 as the size is {x.size(dim)}."

@@ -110,6 +110,11 @@ typedef struct dk_lut {
                           lets heads of a GQA group share K/V tiles inside a workgroup */
   int32_t max_row_entries; /* largest number of entries in one row (0 if unknown); sizes the
                               split-KV decode grid and workspace */
+  int32_t sub_block;   /* 0, or 16 / 32 with entry_width 2 and 64 x 64 tiles: the pattern's own block
+                          size.  The second int of an entry is then a bit mask over the tile's
+                          f x f pattern blocks, f = 64 / sub_block: bit i * f + j set = rows
+                          [i, i+1) * sub_block x columns [j, j+1) * sub_block are attended.  Taken
+                          by the matrix-core kernels only. */
 } dk_lut;
 
 /* Sequence geometry.  With all four pointers NULL every sequence has

@@ -3,7 +3,7 @@ kernels ("auto") against the independent generic fp32 kernels on the same
 inputs, and both against the fp32 dense oracle where the case is small enough.
 The draw covers what selects a kernel variant: heads per kv head (group of 4,
 2, 1 -> head groups, row pairs), head dims (multiples of 8 up to 128 ->
-zero-padded tiles), pattern blocks (64 / 128 / 256 -> split tables), lengths
+zero-padded tiles), pattern blocks (64; 128 / 256 -> split tables; 16 / 32 -> masked tiles), lengths
 that are not multiples of the block, k longer than q, local / vertical
 parameters, dense heads, bf16 / fp16, token or head major layout, forward and
 backward with and without a gradient through LSE."""
@@ -25,10 +25,10 @@ def draw_config(rng):
     ratio = int(rng.choice([1, 1, 2, 4, 8]))
     Hkv = int(rng.choice([1, 2, 3]))
     Hq = Hkv * ratio
-    bs = int(rng.choice([64, 64, 64, 128, 256]))
+    bs = int(rng.choice([64, 64, 64, 128, 256, 16, 32]))
     D = int(rng.choice([128, 128, 64, 96, 48, 80, 112, 32]))
-    nb = int(rng.integers(1, 13)) if bs == 64 else int(rng.integers(1, 6))
-    L = int(rng.integers((nb - 1) * bs + 1, nb * bs + 1))
+    nb = int(rng.integers(1, 13)) if bs <= 64 else int(rng.integers(1, 6))
+    L = int(rng.integers((nb - 1) * max(bs, 64) + 1, nb * max(bs, 64) + 1))
     past = int(rng.choice([0, 0, 0, 64, 37, 200])) if L > 1 else 0
     local = int(rng.integers(1, 5))
     vert = int(rng.integers(1, 7))
@@ -57,7 +57,7 @@ def run_impl(impl, mod, q, k, v, do, dlse, sm, backward):
         ops.set_impl("auto")
 
 
-@pytest.mark.parametrize("seed", range(40))
+@pytest.mark.parametrize("seed", range(60))
 def test_random_config_matches_generic_kernels_and_oracle(seed):
     rng = np.random.default_rng(1000 + seed)
     c = draw_config(rng)
@@ -110,7 +110,7 @@ def _seq_oracle(q, k, v, bm, bs, sm):
     return o[0], lse[0]
 
 
-@pytest.mark.parametrize("seed", range(30))
+@pytest.mark.parametrize("seed", range(40))
 def test_random_inference_config_matches_generic_kernels_and_oracle(seed):
     """Per-sequence lengths: left-padded, right-padded and packed prefill, padded and packed
     single-token decode (split-KV kernels), chunked packed prefill."""
@@ -118,7 +118,7 @@ def test_random_inference_config_matches_generic_kernels_and_oracle(seed):
     ratio = int(rng.choice([1, 2, 4]))
     Hkv = int(rng.choice([1, 2]))
     Hq = Hkv * ratio
-    bs = int(rng.choice([64, 64, 128]))
+    bs = int(rng.choice([64, 64, 128, 16, 32]))
     D = int(rng.choice([128, 64, 96, 40]))
     dtype = torch.bfloat16 if rng.random() < 0.7 else torch.float16
     mode = str(rng.choice(["left", "right", "packed", "packed_decode", "left_decode", "right_decode", "chunked"]))

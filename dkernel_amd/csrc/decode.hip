@@ -47,13 +47,16 @@ struct DecSmem {  // per wave: one 32-key half block of K and of V, plus q of th
 };
 
 // workspace layout: [batch][Hq][max_units][D + 2] floats (O[D] unnormalised, max, sum)
-template <typename T, int D, bool PAD>
+template <typename T, int D, bool PAD, bool SUB>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void decode_partial_kernel(const FwdParams p, float *ws, int unit_blocks,
                                                             int max_units) {
   using M = Mma<T>;
   using vec8 = typename M::vec8;
   using S = DecSmem<D>;
   constexpr int KS = D / 16, DT = D / 32, CPR = D / 8;
+  // SUB: table entries are (column, bit mask over the pattern blocks inside the 64 x 64 tile)
+  static_assert(!SUB || !PAD, "sub-block masks: plain tiles only");
+  constexpr int EW = SUB ? 2 : 1;  // ints per table entry
   extern __shared__ __align__(16) char smem[];
 
   const int unit = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
@@ -74,14 +77,20 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
   if (e0 >= row1) return;  // this row has fewer units
   const int e1 = min(e0 + unit_blocks, row1);
   const int32_t *cols = p.csr.idx + lh * p.csr.idx_sh;
+  // SUB: the query's row of pattern blocks inside its tile selects f of the entry's f x f mask
+  // bits; half block hb & 1 holds key parts [hb & 1, hb & 1 + 1) * f / 2 of them
+  const int lb = SUB ? (p.csr.sub_block == 16 ? 4 : 5) : 6, f = 64 >> lb;
+  const int row_shift = ((pos & 63) >> lb) * f;
+  auto half_bits = [&](int bits, int hb) { return (bits >> (row_shift + (hb & 1) * (f >> 1))) & ((1 << (f >> 1)) - 1); };
   const T *kbase = (const T *)p.k.ptr + sq.b * p.k.sb + kvh * p.k.sh + (int64_t)sq.k_start * p.k.st;
   const T *vbase = (const T *)p.v.ptr + sq.b * p.v.sb + kvh * p.v.sh + (int64_t)sq.k_start * p.v.st;
 
   // half block hb of this unit = keys cols[e0 + hb/2] * 64 + 32 * (hb & 1) + [0, 32)
   constexpr int HCH = 32 * CPR / 64;  // 16-byte chunks per lane per half tile
   uint4 kreg[HCH], vreg[HCH];
-  auto prefetch = [&](int hb, int col) {
+  auto prefetch = [&](int hb, int col, int bits) {
     const int key0 = col * 64 + (hb & 1) * 32;
+    if (SUB && half_bits(bits, hb) == 0) return;  // no attended key in this half: neither read nor used
     if (!PAD && col >= 0 && key0 + 32 <= sq.k_len) {  // whole half inside the sequence: no guards
 #pragma unroll
       for (int c = 0; c < HCH; ++c) {
@@ -104,8 +113,12 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
     }
   };
   // the first K/V request goes out before anything else touches memory
-  int col_cur = scalar_load(cols + e0);
-  prefetch(0, col_cur);
+  int col_cur, bits_cur = 0;
+  if constexpr (SUB)
+    scalar_load2(cols + e0 * EW, cols + e0 * EW + 1, col_cur, bits_cur);
+  else
+    col_cur = scalar_load(cols + e0);
+  prefetch(0, col_cur, bits_cur);
 
   // q of the group's heads -> LDS (row min(m, ratio-1) feeds MFMA column m;
   // columns >= ratio are duplicates whose results are never stored)
@@ -135,24 +148,33 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
 
   for (int hb = 0; hb < nhalf; ++hb) {
     const int col = col_cur;
+    const int hbits = SUB ? half_bits(bits_cur, hb) : 1;
     const int key0 = col * 64 + (hb & 1) * 32;
     // table entry of the next half block (the next block after an odd half)
-    if ((hb & 1) && hb + 1 < nhalf) col_cur = scalar_load(cols + e0 + ((hb + 1) >> 1));
+    if ((hb & 1) && hb + 1 < nhalf) {
+      const int32_t *ent = cols + (e0 + ((hb + 1) >> 1)) * EW;
+      if constexpr (SUB)
+        scalar_load2(ent, ent + 1, col_cur, bits_cur);
+      else
+        col_cur = scalar_load(ent);
+    }
     // The tiles are private to this wave and LDS operations of one wave
     // execute in order, so the previous half block's reads are done; only the
     // compiler must not reorder across these points (a memory fence would
     // also drain the global prefetch issued next).
     asm volatile("" ::: "memory");
+    if (hbits != 0) {  // (a half without attended keys was not read)
 #pragma unroll
-    for (int c = 0; c < HCH; ++c) {
-      const int idx = lane + c * 64;
-      const int r = idx / CPR, ch = idx % CPR;
-      *reinterpret_cast<uint4 *>(ks_ + r * S::kStride + ch * 16) = kreg[c];
-      *reinterpret_cast<uint4 *>(vs_ + r * S::kStride + ch * 16) = vreg[c];
+      for (int c = 0; c < HCH; ++c) {
+        const int idx = lane + c * 64;
+        const int r = idx / CPR, ch = idx % CPR;
+        *reinterpret_cast<uint4 *>(ks_ + r * S::kStride + ch * 16) = kreg[c];
+        *reinterpret_cast<uint4 *>(vs_ + r * S::kStride + ch * 16) = vreg[c];
+      }
     }
     asm volatile("" ::: "memory");
-    if (hb + 1 < nhalf) prefetch(hb + 1, col_cur);
-    if (col < 0 || key0 >= sq.k_len || (p.causal && key0 > pos)) continue;
+    if (hb + 1 < nhalf) prefetch(hb + 1, col_cur, bits_cur);
+    if (hbits == 0 || col < 0 || key0 >= sq.k_len || (p.causal && key0 > pos)) continue;
 
     floatx16 sacc;
 #pragma unroll
@@ -172,6 +194,10 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       float sv = sacc[r] * p.scale_log2;
+      if constexpr (SUB) {
+        // key 8 (r / 4) + 4 g + r % 4 of the half: the last two terms stay inside a part of >= 16 keys
+        if (!((hbits >> (((r >> 2) * 8) >> lb)) & 1)) sv = -INFINITY;
+      }
       if (need_mask) {
         const int key = key0 + (r >> 2) * 8 + g * 4 + (r & 3);
         if (key >= sq.k_len || (p.causal && key > pos)) sv = -INFINITY;
@@ -301,7 +327,8 @@ bool decode_supported(const FwdParams &p, int dtype) {
   const bool shared_row = p.csr.num_heads == 1 || (p.csr.num_heads == p.Hkv && p.Hkv != p.Hq) || ratio == 1 ||
                           (p.csr.num_heads == p.Hq && p.csr.group % ratio == 0);
   return (dtype == DK_BF16 || dtype == DK_F16) && mfma_head_dim_ok(p.D) && p.csr.block_rows == 64 &&
-         p.csr.block_cols == 64 && p.csr.entry_width == 1 && p.vec_ok &&
+         p.csr.block_cols == 64 && p.vec_ok &&
+         (p.csr.entry_width == 1 || (p.csr.sub_block != 0 && (p.D == 64 || p.D == 128))) &&
          (p.seqs.packed ? (p.seqs.packed & 2) != 0 : p.seqs.max_q_len == 1) && ratio <= 32 && shared_row && p.causal;
 }
 
@@ -309,12 +336,12 @@ size_t decode_workspace_bytes(const FwdParams &p) {
   return (size_t)p.seqs.batch * p.Hq * decode_max_units(p) * (mfma_tile_width(p.D) + 2) * sizeof(float);
 }
 
-template <typename T, int D, bool PAD>
+template <typename T, int D, bool PAD, bool SUB>
 static int launch_decode_td(const FwdParams &p, float *ws, hipStream_t stream) {
   const int smem = DecSmem<D>::wave_bytes(p.Hq / p.Hkv);
   const int unit_blocks = decode_unit_blocks(), max_units = decode_max_units(p);
   DK_REQUIRE(max_units <= 65535, "too many decode units");
-  hipLaunchKernelGGL((decode_partial_kernel<T, D, PAD>), dim3(max_units, p.Hkv, p.seqs.batch), dim3(64), smem, stream,
+  hipLaunchKernelGGL((decode_partial_kernel<T, D, PAD, SUB>), dim3(max_units, p.Hkv, p.seqs.batch), dim3(64), smem, stream,
                      p, ws, unit_blocks, max_units);
   DK_HIP_CHECK(hipGetLastError());
   hipLaunchKernelGGL((decode_combine_kernel<T, D, PAD>), dim3(p.Hq, p.seqs.batch), dim3(64), 0, stream, p, ws,
@@ -326,9 +353,13 @@ static int launch_decode_td(const FwdParams &p, float *ws, hipStream_t stream) {
 // head dims below the tile width (64 or 128) run the zero-padded instantiation
 template <typename T>
 static int launch_decode_t(const FwdParams &p, float *ws, hipStream_t stream) {
-  if (p.D == 128) return launch_decode_td<T, 128, false>(p, ws, stream);
-  if (p.D == 64) return launch_decode_td<T, 64, false>(p, ws, stream);
-  return p.D > 64 ? launch_decode_td<T, 128, true>(p, ws, stream) : launch_decode_td<T, 64, true>(p, ws, stream);
+  if (p.csr.sub_block)  // entries carry a bit mask over the pattern's 16- or 32-token blocks
+    return p.D == 128 ? launch_decode_td<T, 128, false, true>(p, ws, stream)
+                      : launch_decode_td<T, 64, false, true>(p, ws, stream);
+  if (p.D == 128) return launch_decode_td<T, 128, false, false>(p, ws, stream);
+  if (p.D == 64) return launch_decode_td<T, 64, false, false>(p, ws, stream);
+  return p.D > 64 ? launch_decode_td<T, 128, true, false>(p, ws, stream)
+                  : launch_decode_td<T, 64, true, false>(p, ws, stream);
 }
 
 int launch_decode(const FwdParams &p, int dtype, void *workspace, size_t workspace_bytes, hipStream_t stream) {

@@ -323,7 +323,7 @@ def test_packed_varlen_prefill_and_decode(impl, D, bs):
     qd = torch.randn(len(lens), Hq, D, generator=g).to(torch.bfloat16)
     outd = mod(qd.to(DEV), k.to(DEV), v.to(DEV), sm, cu_seqlen_k=cu.to(DEV))
     # one query token per packed sequence takes the split-KV decode kernel whenever 64-tiles apply
-    assert (ops.last_fwd_workspace_bytes > 0) == (impl == "auto" and bs != 32)
+    assert (ops.last_fwd_workspace_bytes > 0) == (impl == "auto")
     for i, l in enumerate(lens):
         s, e = int(cu[i]), int(cu[i + 1])
         ro, _ = _seq_oracle(qd[i:i + 1], k[s:e], v[s:e], bm, bs, sm)

@@ -112,7 +112,7 @@ static int make_bwd_params(const dk_bwd_args *a, BwdParams &p, bool &empty) {
   if (rc) return rc;
   rc = check_lut(a->csc, "csc", a->num_q_heads, a->num_kv_heads);
   if (rc) return rc;
-  DK_REQUIRE(a->csc.entry_width == 1, "csc table cannot carry values");
+  DK_REQUIRE(a->csc.entry_width == 1 || a->csc.sub_block != 0, "csc table cannot carry values other than sub-block masks");
   DK_REQUIRE((int64_t)a->csr.num_rows * a->csr.block_rows >= a->seqs.max_k_len,
              "Input length %d is larger than the maximum length allowed", a->seqs.max_k_len);
   if (a->seqs.batch == 0 || a->seqs.max_q_len == 0) {

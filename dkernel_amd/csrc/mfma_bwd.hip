@@ -43,7 +43,7 @@ struct BoolConst {
 // ---------------------------------------------------------------------------
 // dQ pass
 // ---------------------------------------------------------------------------
-template <typename T, int D, bool PAD>
+template <typename T, int D, bool PAD, bool SUB>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void mfma_dq_kernel(const BwdParams p,
                                                                                                    int tiles_y) {
   using M = Mma<T>;
@@ -52,6 +52,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   constexpr int NT = 256;
   constexpr int KS = D / 16, DT = D / 32;
   constexpr int STAGE = 2 * TL::kBytes;
+  // SUB: table entries are (column, bit mask over the pattern blocks inside the 64 x 64 tile)
+  static_assert(!SUB || !PAD, "sub-block masks: plain tiles only");
+  constexpr int EW = SUB ? 2 : 1;  // ints per table entry
   extern __shared__ __align__(16) char smem[];
 
   const SeqInfo sq = load_seq(p.seqs, blockIdx.z, p.causal);
@@ -141,8 +144,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   // Table entries: block e in col_cur (scalar register); block e + 1 is requested one block
   // early as a vector load (col_pending) and first used behind the next tile wait, so that no
   // table read ever stalls the loop.
-  int col_cur = e0 < e1 ? scalar_load(cols + e0) : 0;
-  int col_pending = e0 + 1 < e1 ? cols[e0 + 1] : 0;
+  int col_cur = e0 < e1 ? scalar_load(cols + e0 * EW) : 0;
+  int col_pending = e0 + 1 < e1 ? cols[(e0 + 1) * EW] : 0;
+  int bits_cur = 0, bits_pending = 0;  // SUB: the entry's mask, carried like the column
+  if constexpr (SUB) {
+    bits_cur = e0 < e1 ? scalar_load(cols + e0 * EW + 1) : 0;
+    bits_pending = e0 + 1 < e1 ? cols[(e0 + 1) * EW + 1] : 0;
+  }
   if (e0 < e1) issue(col_cur, 0);  // the first tiles are on their way while the row data is fetched
 
   // Q and dO fragments, lse in the log2 domain, and delta = rowsum(O * dO) - dLSE, which this
@@ -165,10 +173,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   auto block_step = [&](int e, auto stage_tag) {
     constexpr int stage = decltype(stage_tag)::value;
     const int col = col_cur;
+    const int bits = bits_cur;
     wait_tile_loads();
     __syncthreads();  // tile e is visible; every wave is done with the other stage
     const int col_next = __builtin_amdgcn_readfirstlane(col_pending);  // landed before the tile did
-    if (e + 2 < e1) col_pending = cols[e + 2];
+    if constexpr (SUB) bits_cur = __builtin_amdgcn_readfirstlane(bits_pending);
+    if (e + 2 < e1) {
+      col_pending = cols[(e + 2) * EW];
+      if constexpr (SUB) bits_pending = cols[(e + 2) * EW + 1];
+    }
     if (e + 1 < e1) issue(col_next, stage ^ 1);
     col_cur = col_next;
     const int key0 = col * 64 + kh * 32;  // first key of this wave's half
@@ -212,6 +225,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       for (int r = 0; r < 16; ++r) {
         const int key = key0 + (r >> 2) * 8 + g * 4 + (r & 3);
         s[r] = key > lim ? 0.f : s[r];
+      }
+    }
+    if constexpr (SUB) {
+      // pattern blocks of the tile that this row does not attend: bit (row part) * f + (key part)
+      const int lb = p.csr.sub_block == 16 ? 4 : 5, f = 64 >> lb;
+      const int full = f == 4 ? 0xffff : 0xf;
+      if ((bits & full) != full) {  // wave-uniform
+        const int row_bits = bits >> (((rh * 32 + m) >> lb) * f);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          // key kh 32 + 8 (r / 4) + 4 g + r % 4: the last two terms stay inside a part of >= 16 keys
+          const int key_part = (kh * 32 + (r >> 2) * 8) >> lb;
+          s[r] = ((row_bits >> key_part) & 1) ? s[r] : 0.f;
+        }
       }
     }
 #pragma unroll
@@ -290,7 +317,7 @@ struct DkdvSmem {
   static constexpr int kBytes = kLoop > kRed ? kLoop : kRed;
 };
 
-template <typename T, int D, bool PAD>
+template <typename T, int D, bool PAD, bool SUB>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void mfma_dkdv_kernel(const BwdParams p, int head_split) {
   using M = Mma<T>;
   using vec8 = typename M::vec8;
@@ -299,6 +326,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   constexpr int NT = 512;
   constexpr int KS = D / 16, DT = D / 32;
   constexpr int LPT = 2 * TileLoader<D, NT>::kChunks + 1;  // load instructions per wave per block
+  // SUB: table entries are (row block, bit mask over the pattern blocks inside the 64 x 64 tile)
+  static_assert(!SUB || !PAD, "sub-block masks: plain tiles only");
+  constexpr int EW = SUB ? 2 : 1;  // ints per table entry
   extern __shared__ __align__(16) char smem[];
 
   const SeqInfo sq = load_seq(p.seqs, blockIdx.z, p.causal);
@@ -357,7 +387,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     if (cb < p.csc.num_rows)
       scalar_load2(p.csc.ptr + lh * p.csc.ptr_sh + cb, p.csc.ptr + lh * p.csc.ptr_sh + cb + 1, e0, e1);
     const int nblk = e1 - e0;
-    const int32_t *rows = p.csc.idx + lh * p.csc.idx_sh + e0;
+    const int32_t *rows = p.csc.idx + lh * p.csc.idx_sh + e0 * EW;
     const T *qbase = (const T *)p.q.ptr + sq.b * p.q.sb + h * p.q.sh;
     const T *dobase = (const T *)p.dout.ptr + sq.b * p.dout.sb + h * p.dout.sh;
     const float *lsebase = p.lse.ptr + sq.b * p.lse.sb + h * p.lse.sh;
@@ -430,7 +460,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     static_assert(S::kAhead == 2, "the first two table entries are read together");
     if (nblk > 0) {
       int r0, r1;
-      scalar_load2(rows, rows + (nblk > 1 ? 1 : 0), r0, r1);  // one round trip for both
+      scalar_load2(rows, rows + (nblk > 1 ? EW : 0), r0, r1);  // one round trip for both
       for (int i = 0; i < S::kAhead && issued < nblk; ++i, ++issued) {
         exact = issue(i == 0 ? r0 : r1, iq, ido) && exact;
         iq = iq + 1 == S::kQStages ? 0 : iq + 1;
@@ -443,14 +473,18 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       wait_tiles_ahead<LPT>(exact ? issued - t - 1 : 0);
       __syncthreads();  // block t is visible, so is P of block t - 1; the stages of block t - 2 are free
       if (issued < nblk) {
-        exact = issue(scalar_load(rows + issued), iq, ido) && exact;
+        exact = issue(scalar_load(rows + issued * EW), iq, ido) && exact;
         iq = iq + 1 == S::kQStages ? 0 : iq + 1;
         ido = ido + 1 == S::kDoStages ? 0 : ido + 1;
         ++issued;
       }
       const char *qs_ = smem + S::kQ + cq * TL::kBytes, *dos_ = smem + S::kDo + cdo * TL::kBytes;
       if constexpr (!kDp) {
-        const int rbq = scalar_load(rows + t);
+        int rbq, bits = 0;
+        if constexpr (SUB)
+          scalar_load2(rows + t * EW, rows + t * EW + 1, rbq, bits);
+        else
+          rbq = scalar_load(rows + t);
         const int pos0 = rbq * 64 + mh * 32;  // first q position of this wave's half
         const float *lse_s = reinterpret_cast<const float *>(smem + S::kVec + cq * 512);
         // S = Q K^T : rows = 32 q positions, cols = 32 keys
@@ -492,6 +526,20 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         if (edge) {
 #pragma unroll
           for (int r = 0; r < 16; ++r) sc[r] = kcmp > (r >> 2) * 8 + g * 4 + (r & 3) ? 0.f : sc[r];
+        }
+        if constexpr (SUB) {
+          // pattern blocks of the tile that are not attended: bit (row part) * f + (key part); this
+          // lane's key is nh 32 + n, register r is q row mh 32 + 8 (r / 4) + 4 g + r % 4
+          const int lb = p.csc.sub_block == 16 ? 4 : 5, f = 64 >> lb;
+          const int full = f == 4 ? 0xffff : 0xf;
+          if ((bits & full) != full) {  // wave-uniform
+            const int key_bits = bits >> ((nh * 32 + n) >> lb);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const int row_part = (mh * 32 + (r >> 2) * 8) >> lb;
+              sc[r] = ((key_bits >> (row_part * f)) & 1) ? sc[r] : 0.f;
+            }
+          }
         }
 #pragma unroll
         for (int r4 = 0; r4 < 4; ++r4)
@@ -589,22 +637,30 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
 // Explicit instantiations: with only the implicit ones the fp16 host stubs of
 // these kernels are not emitted by this compiler version.
-template __global__ void mfma_dq_kernel<bf16_t, 128, false>(const BwdParams, int);
-template __global__ void mfma_dq_kernel<bf16_t, 128, true>(const BwdParams, int);
-template __global__ void mfma_dq_kernel<bf16_t, 64, false>(const BwdParams, int);
-template __global__ void mfma_dq_kernel<bf16_t, 64, true>(const BwdParams, int);
-template __global__ void mfma_dq_kernel<f16_t, 128, false>(const BwdParams, int);
-template __global__ void mfma_dq_kernel<f16_t, 128, true>(const BwdParams, int);
-template __global__ void mfma_dq_kernel<f16_t, 64, false>(const BwdParams, int);
-template __global__ void mfma_dq_kernel<f16_t, 64, true>(const BwdParams, int);
-template __global__ void mfma_dkdv_kernel<bf16_t, 128, false>(const BwdParams, int);
-template __global__ void mfma_dkdv_kernel<bf16_t, 128, true>(const BwdParams, int);
-template __global__ void mfma_dkdv_kernel<bf16_t, 64, false>(const BwdParams, int);
-template __global__ void mfma_dkdv_kernel<bf16_t, 64, true>(const BwdParams, int);
-template __global__ void mfma_dkdv_kernel<f16_t, 128, false>(const BwdParams, int);
-template __global__ void mfma_dkdv_kernel<f16_t, 128, true>(const BwdParams, int);
-template __global__ void mfma_dkdv_kernel<f16_t, 64, false>(const BwdParams, int);
-template __global__ void mfma_dkdv_kernel<f16_t, 64, true>(const BwdParams, int);
+template __global__ void mfma_dq_kernel<bf16_t, 128, false, false>(const BwdParams, int);
+template __global__ void mfma_dq_kernel<bf16_t, 128, true, false>(const BwdParams, int);
+template __global__ void mfma_dq_kernel<bf16_t, 128, false, true>(const BwdParams, int);
+template __global__ void mfma_dq_kernel<bf16_t, 64, false, false>(const BwdParams, int);
+template __global__ void mfma_dq_kernel<bf16_t, 64, true, false>(const BwdParams, int);
+template __global__ void mfma_dq_kernel<bf16_t, 64, false, true>(const BwdParams, int);
+template __global__ void mfma_dq_kernel<f16_t, 128, false, false>(const BwdParams, int);
+template __global__ void mfma_dq_kernel<f16_t, 128, true, false>(const BwdParams, int);
+template __global__ void mfma_dq_kernel<f16_t, 128, false, true>(const BwdParams, int);
+template __global__ void mfma_dq_kernel<f16_t, 64, false, false>(const BwdParams, int);
+template __global__ void mfma_dq_kernel<f16_t, 64, true, false>(const BwdParams, int);
+template __global__ void mfma_dq_kernel<f16_t, 64, false, true>(const BwdParams, int);
+template __global__ void mfma_dkdv_kernel<bf16_t, 128, false, false>(const BwdParams, int);
+template __global__ void mfma_dkdv_kernel<bf16_t, 128, true, false>(const BwdParams, int);
+template __global__ void mfma_dkdv_kernel<bf16_t, 128, false, true>(const BwdParams, int);
+template __global__ void mfma_dkdv_kernel<bf16_t, 64, false, false>(const BwdParams, int);
+template __global__ void mfma_dkdv_kernel<bf16_t, 64, true, false>(const BwdParams, int);
+template __global__ void mfma_dkdv_kernel<bf16_t, 64, false, true>(const BwdParams, int);
+template __global__ void mfma_dkdv_kernel<f16_t, 128, false, false>(const BwdParams, int);
+template __global__ void mfma_dkdv_kernel<f16_t, 128, true, false>(const BwdParams, int);
+template __global__ void mfma_dkdv_kernel<f16_t, 128, false, true>(const BwdParams, int);
+template __global__ void mfma_dkdv_kernel<f16_t, 64, false, false>(const BwdParams, int);
+template __global__ void mfma_dkdv_kernel<f16_t, 64, true, false>(const BwdParams, int);
+template __global__ void mfma_dkdv_kernel<f16_t, 64, false, true>(const BwdParams, int);
 
 // Sum of the per-q-head dK / dV partials over each kv group (head_split mode).  One thread
 // per 8 head dims of one (batch, kv head, key): blockIdx.y = 0 sums dK, 1 sums dV.
@@ -648,23 +704,25 @@ size_t mfma_bwd_workspace_bytes(const BwdParams &p) {
 
 bool mfma_bwd_supported(const BwdParams &p, int dtype) {
   return (dtype == DK_BF16 || dtype == DK_F16) && mfma_head_dim_ok(p.D) && p.csr.block_rows == 64 &&
-         p.csr.block_cols == 64 && p.csr.entry_width == 1 && p.csc.block_rows == 64 && p.csc.block_cols == 64 &&
+         p.csr.block_cols == 64 && p.csr.sub_block == p.csc.sub_block &&
+         (p.csr.sub_block ? (p.D == 64 || p.D == 128) : (p.csr.entry_width == 1 && p.csc.entry_width == 1)) &&
+         p.csc.block_rows == 64 && p.csc.block_cols == 64 &&
          p.vec_ok;
 }
 
-template <typename T, int D, bool PAD>
+template <typename T, int D, bool PAD, bool SUB>
 static int launch_bwd_td(const BwdParams &p, void *workspace, size_t workspace_bytes, hipStream_t stream) {
   const SeqView &s = p.seqs;
   constexpr int smem_dq = 2 * 2 * Tile<D>::kBytes;
   constexpr int smem_dkdv = DkdvSmem<D>::kBytes;
-  DK_ALLOW_DYNAMIC_LDS((mfma_dq_kernel<T, D, PAD>), smem_dq);
-  DK_ALLOW_DYNAMIC_LDS((mfma_dkdv_kernel<T, D, PAD>), smem_dkdv);
+  DK_ALLOW_DYNAMIC_LDS((mfma_dq_kernel<T, D, PAD, SUB>), smem_dq);
+  DK_ALLOW_DYNAMIC_LDS((mfma_dkdv_kernel<T, D, PAD, SUB>), smem_dkdv);
   const int past = p.causal ? s.max_k_len - s.max_q_len : 0;
   const int tiles = (past + s.max_q_len - 1) / 64 - past / 64 + 1;
   const int cblocks = cdiv(s.max_k_len, 64);
   DK_REQUIRE(tiles <= 65535 && cblocks <= 65535, "sequence too long for one launch");
   // dQ first: it also writes delta, which the dK/dV pass reads
-  hipLaunchKernelGGL((mfma_dq_kernel<T, D, PAD>), dim3(p.Hq, tiles, s.batch), dim3(256), smem_dq, stream, p, tiles);
+  hipLaunchKernelGGL((mfma_dq_kernel<T, D, PAD, SUB>), dim3(p.Hq, tiles, s.batch), dim3(256), smem_dq, stream, p, tiles);
   DK_HIP_CHECK(hipGetLastError());
   // With several q heads per kv head a workgroup per kv head walks all of them, and the longest
   // column (a vertical one near the start: every later q block, times the group size) alone
@@ -677,7 +735,7 @@ static int launch_bwd_td(const BwdParams &p, void *workspace, size_t workspace_b
     float *part_k = (float *)workspace, *part_v = part_k + (int64_t)s.batch * p.Hq * keys * p.D;
     pp.dk = TensorView{part_k, p.Hq * keys * p.D, keys * p.D, p.D};
     pp.dv = TensorView{part_v, p.Hq * keys * p.D, keys * p.D, p.D};
-    hipLaunchKernelGGL((mfma_dkdv_kernel<T, D, PAD>), dim3(p.Hq, cblocks, s.batch), dim3(512), smem_dkdv, stream, pp, 1);
+    hipLaunchKernelGGL((mfma_dkdv_kernel<T, D, PAD, SUB>), dim3(p.Hq, cblocks, s.batch), dim3(512), smem_dkdv, stream, pp, 1);
     DK_HIP_CHECK(hipGetLastError());
     const int64_t total = (int64_t)s.batch * p.Hkv * keys * (p.D / 8);
     hipLaunchKernelGGL((dkdv_group_sum_kernel<T>), dim3((unsigned)cdiv64(total, 256), 2), dim3(256), 0, stream, part_k,
@@ -685,7 +743,7 @@ static int launch_bwd_td(const BwdParams &p, void *workspace, size_t workspace_b
     DK_HIP_CHECK(hipGetLastError());
     return DK_OK;
   }
-  hipLaunchKernelGGL((mfma_dkdv_kernel<T, D, PAD>), dim3(p.Hkv, cblocks, s.batch), dim3(512), smem_dkdv, stream, p, 0);
+  hipLaunchKernelGGL((mfma_dkdv_kernel<T, D, PAD, SUB>), dim3(p.Hkv, cblocks, s.batch), dim3(512), smem_dkdv, stream, p, 0);
   DK_HIP_CHECK(hipGetLastError());
   return DK_OK;
 }
@@ -693,10 +751,13 @@ static int launch_bwd_td(const BwdParams &p, void *workspace, size_t workspace_b
 // head dims below the tile width (64 or 128) run the zero-padded instantiation
 template <typename T>
 static int launch_bwd_t(const BwdParams &p, void *ws, size_t ws_bytes, hipStream_t stream) {
-  if (p.D == 128) return launch_bwd_td<T, 128, false>(p, ws, ws_bytes, stream);
-  if (p.D == 64) return launch_bwd_td<T, 64, false>(p, ws, ws_bytes, stream);
-  return p.D > 64 ? launch_bwd_td<T, 128, true>(p, ws, ws_bytes, stream)
-                  : launch_bwd_td<T, 64, true>(p, ws, ws_bytes, stream);
+  if (p.csr.sub_block)  // entries carry a bit mask over the pattern's 16- or 32-token blocks
+    return p.D == 128 ? launch_bwd_td<T, 128, false, true>(p, ws, ws_bytes, stream)
+                      : launch_bwd_td<T, 64, false, true>(p, ws, ws_bytes, stream);
+  if (p.D == 128) return launch_bwd_td<T, 128, false, false>(p, ws, ws_bytes, stream);
+  if (p.D == 64) return launch_bwd_td<T, 64, false, false>(p, ws, ws_bytes, stream);
+  return p.D > 64 ? launch_bwd_td<T, 128, true, false>(p, ws, ws_bytes, stream)
+                  : launch_bwd_td<T, 64, true, false>(p, ws, ws_bytes, stream);
 }
 
 int launch_mfma_bwd(const BwdParams &p, int dtype, void *workspace, size_t workspace_bytes, hipStream_t stream) {

@@ -81,7 +81,7 @@ class SparseAttention(torch.nn.Module):
         # tables split to that tile, unless the caller fixes the tile sizes.
         split_for_kernels = block_m is None and block_n is None and block_size > _KERNEL_TILE
         # ... and patterns with smaller blocks on tile tables whose entries carry a bit mask over
-        # the pattern blocks inside the tile (forward only; backward keeps the tables above)
+        # the pattern blocks inside the tile
         mask_for_kernels = block_m is None and block_n is None and block_size < _KERNEL_TILE
         if block_m is None:
             block_m = max(block_size, 64) if causal else block_size
@@ -156,15 +156,18 @@ class SparseAttention(torch.nn.Module):
 
         self.mask_tile = None
         if mask_for_kernels:
-            m_csr, _ = masked_tile_tables(block_size, sparse_pattern, _KERNEL_TILE)
-            m_csr = list(m_csr)
+            m_csr, m_csc = masked_tile_tables(block_size, sparse_pattern, _KERNEL_TILE)
+            m_csr, m_csc = list(m_csr), list(m_csc)
             if m_csr[0].size(0) == 1:
                 m_csr = [zero_stride(x) for x in m_csr]
+                m_csc = [zero_stride(x) for x in m_csc]
             crow = m_csr[0]
             self.mask_tile = _KERNEL_TILE
             self.mask_lut_max_row = int((crow[:, 1:] - crow[:, :-1]).max()) if crow.size(1) > 1 else 0
             self.register_buffer("masked_csr_crow", m_csr[0].to(torch.int32), persistent=False)
             self.register_buffer("masked_csr_col", m_csr[1].to(torch.int32), persistent=False)
+            self.register_buffer("masked_csc_ccol", m_csc[0].to(torch.int32), persistent=False)
+            self.register_buffer("masked_csc_row", m_csc[1].to(torch.int32), persistent=False)
 
     def forward(self,
                 q: Tensor,
@@ -205,8 +208,10 @@ class SparseAttention(torch.nn.Module):
             layout_csc = (self.layout_csc_ccol, self.layout_csc_row, self.block_m2, self.block_n2)
         if self.mask_tile is not None:
             # (crow, (col, mask), tile rows, tile cols, pattern block size), longest row
-            kwargs["masked_fwd_layout"] = ((self.masked_csr_crow, self.masked_csr_col, self.mask_tile,
-                                            self.mask_tile, self.block_size), self.mask_lut_max_row)
+            kwargs["masked_layouts"] = ((self.masked_csr_crow, self.masked_csr_col, self.mask_tile,
+                                         self.mask_tile, self.block_size),
+                                        (self.masked_csc_ccol, self.masked_csc_row, self.mask_tile,
+                                         self.mask_tile, self.block_size), self.mask_lut_max_row)
         output, lse = _sparse_attention.apply(
             q, k, v, sm_scale, layout_csr, layout_csc,
             self.seq_dim, inf_kwargs, kwargs)

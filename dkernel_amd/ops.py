@@ -35,15 +35,18 @@ def set_impl(name: str) -> None:
     _impl = _IMPL[name]
 
 
-def _matrix_core_forward_applies(q: Tensor, k: Tensor, v: Tensor, out: Optional[Tensor]) -> bool:
-    """Whether dk_fwd will run these inputs on the matrix-core kernels with a masked tile table:
+def _matrix_core_applies(*xs: Optional[Tensor]) -> bool:
+    """Whether dk_fwd / dk_bwd will run these tensors on the matrix-core kernels with a masked tile table:
     16-bit floats, head_dim 64 or 128, 16-byte aligned rows (the library's own conditions; it
     fails loudly if they were judged wrong here)."""
+    q = xs[0]
     if _impl == _lib.DK_IMPL_GENERIC or q.dtype not in (torch.bfloat16, torch.float16):
         return False
     if q.size(-1) not in (64, 128):
         return False
-    for x in (q, k, v) + ((out,) if out is not None else ()):
+    for x in xs:
+        if x is None:
+            continue
         if x.stride(-1) != 1 or x.data_ptr() % 16 or any(st % 8 for st in x.stride()[:-1]):
             return False
     return True
@@ -217,8 +220,12 @@ def _backward(ctx, do: Tensor, dlse: Optional[Tensor],
     else:
         args.dlse = _rowvec(None)
     args.delta = delta.data_ptr()
-    args.csr = _lut(ctx.layout_csr, q.device, ctx.lut_group)
-    args.csc = _lut(ctx.layout_csc, q.device, ctx.lut_group)
+    layout_csr, layout_csc = ctx.layout_csr, ctx.layout_csc
+    masked = getattr(ctx, "masked_layouts", None)
+    if masked is not None and _matrix_core_applies(q, k, v, o, do, dq, dk, dv):
+        layout_csr, layout_csc = masked[0], masked[1]
+    args.csr = _lut(layout_csr, q.device, ctx.lut_group)
+    args.csc = _lut(layout_csc, q.device, ctx.lut_group)
     args.seqs = _lib.Seqs(B, Lq, k.size(seq_dim), 0, None, None, None, None)
     args.num_q_heads, args.num_kv_heads, args.head_dim = Hq, k.size(hdim), q.size(-1)
     args.dtype, args.causal, args.impl = _DTYPES[q.dtype], int(bool(ctx.causal)), _impl
@@ -412,11 +419,12 @@ class _sparse_attention(torch.autograd.Function):
              f"but the number of heads in the sparse pattern is {layout_csr_crow.size(0)}")
         sm_scale = sm_scale or 1. / math.sqrt(float(q.size(-1)))
 
-        # Patterns with blocks below the kernel tile: the forward runs on the masked tile table
-        # whenever the matrix-core kernels take these inputs; backward keeps the module's tables.
-        masked = kwargs.get("masked_fwd_layout", None)
-        if masked is not None and _matrix_core_forward_applies(q, k, v, kwargs.get("out", None)):
-            layout_csr, lut_max_row = masked
+        # Patterns with blocks below the kernel tile run on the masked tile tables whenever the
+        # matrix-core kernels take these inputs (the backward decides again for its own tensors).
+        masked = kwargs.get("masked_layouts", None)
+        ctx.masked_layouts = masked
+        if masked is not None and _matrix_core_applies(q, k, v, kwargs.get("out", None)):
+            layout_csr, _, lut_max_row = masked
         else:
             lut_max_row = kwargs.get("lut_max_row", 0)
 

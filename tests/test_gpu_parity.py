@@ -121,9 +121,10 @@ def test_matrix_core_kernels_take_padded_dims_and_split_blocks():
     try:
         run_fwd_bwd(1, 8, 2, 512, 96, torch.bfloat16, 64, 2, 4)
         run_fwd_bwd(1, 4, 4, 512, 48, torch.float16, 128, 1, 2)
-        # blocks of 16 / 32: forward on tile tables with a bit mask per entry
-        run_fwd_bwd(2, 8, 2, 1000, 128, torch.bfloat16, 16, 5, 7, backward=False)
-        run_fwd_bwd(1, 4, 4, 777, 64, torch.float16, 32, 3, 3, backward=False)
+        # blocks of 16 / 32: tile tables with a bit mask per entry, forward and backward
+        run_fwd_bwd(2, 8, 2, 1000, 128, torch.bfloat16, 16, 5, 7)
+        run_fwd_bwd(1, 4, 4, 777, 64, torch.float16, 32, 3, 3)
+        run_fwd_bwd(1, 2, 2, 512, 128, torch.bfloat16, 16, 3, 9, causal=False)
         with pytest.raises(Exception, match="no MFMA"):
             run_fwd_bwd(1, 2, 2, 256, 160, torch.bfloat16, 64, 2, 4)
     finally:

@@ -174,6 +174,40 @@ def test_large_blocks_get_split_kernel_tables(bs, causal):
     assert LocalStrideSparseAttention(H, L, 64, 2, 4, causal=causal).kernel_tile is None
 
 
+@pytest.mark.parametrize("bs,causal", [(16, True), (32, True), (16, False)])
+def test_small_blocks_get_masked_tile_tables(bs, causal):
+    """Blocks below the 64 x 64 kernel tile: one table entry per tile that holds any active
+    block, with a bit mask (bit i * f + j: row part i, column part j) that reconstructs the
+    pattern exactly, as CSR and CSC; the layout_* buffers keep the reference's shapes."""
+    L, H = 1000, 4
+    m = LocalStrideSparseAttention(H, L, bs, 3, 5, causal=causal)
+    assert m.mask_tile == 64 and m.kernel_tile is None
+    assert (m.block_m, m.block_n) == ((64, bs) if causal else (bs, bs))
+    pattern = np.asarray(OL.block_mask(H, 1024, bs, 3, 5, causal=causal)) != 0
+    f = 64 // bs
+
+    def rebuild(ptr, idx, transposed):
+        ptr, idx = ptr.numpy(), idx.numpy()
+        out = np.zeros((ptr.shape[0], 1024 // bs, 1024 // bs), dtype=bool)
+        for h in range(ptr.shape[0]):
+            for a in range(ptr.shape[1] - 1):
+                for e in range(ptr[h, a], ptr[h, a + 1]):
+                    b, bits = idx[h, e]
+                    r, c = (b, a) if transposed else (a, b)
+                    assert bits != 0
+                    for i in range(f):
+                        for j in range(f):
+                            out[h, r * f + i, c * f + j] = (bits >> (i * f + j)) & 1
+        return out
+    want = np.broadcast_to(pattern, (m.masked_csr_crow.shape[0],) + pattern.shape[1:])
+    assert np.array_equal(rebuild(m.masked_csr_crow, m.masked_csr_col, False), want)
+    assert np.array_equal(rebuild(m.masked_csc_ccol, m.masked_csc_row, True), want)
+    crow = m.masked_csr_crow.numpy()
+    assert m.mask_lut_max_row == int((crow[:, 1:] - crow[:, :-1]).max())
+    # explicit tile sizes are honoured as given
+    assert LocalStrideSparseAttention(H, L, bs, 3, 5, causal=causal, block_m=bs, block_n=bs).mask_tile is None
+
+
 def test_cpu_tensors_are_refused_loudly():
     m = LocalStrideSparseAttention(2, 128, 64, 1, 2)
     x = torch.zeros(1, 128, 2, 64)

@@ -8,8 +8,10 @@ and need no GPU.
 from __future__ import annotations
 
 import ctypes as C
+from collections import namedtuple
 from typing import Optional, Tuple, Union
 
+import numpy as np
 import torch
 from torch import Tensor
 
@@ -19,6 +21,7 @@ __all__ = [
     "get_sparse_attn_mask", "dense_to_crow_col", "dense_to_ccol_row", "crow_col_to_dense",
     "ccol_row_to_dense", "merge_split_fwd_kernel_blocks", "is_kv_cache_efficient",
     "verify_sparse_pattern", "is_causal", "zero_stride", "multiple_of", "get_q_block_ids", "cdiv",
+    "to_csr", "is_hip", "split_tile_tables", "masked_tile_tables",
 ]
 
 
@@ -28,6 +31,26 @@ def cdiv(a: int, b: int) -> int:
 
 def _ptr(t: Tensor):
     return C.c_void_p(t.data_ptr())
+
+
+_CsrMatrix = namedtuple("csr_matrix", ("indptr", "indices", "data"))
+
+
+def to_csr(mat: np.ndarray) -> _CsrMatrix:
+    """CSR triple (indptr, indices, data) of one 2-D numpy matrix, int32
+    indices.  Reference: dkernel/utils.py:19-24."""
+    mat = np.asarray(mat)
+    nz = mat != 0
+    rows, cols = np.nonzero(nz)
+    indptr = np.zeros(mat.shape[0] + 1, dtype=np.int32)
+    np.cumsum(np.bincount(rows, minlength=mat.shape[0]), out=indptr[1:])
+    return _CsrMatrix(indptr, cols.astype(np.int32), mat[nz])
+
+
+def is_hip() -> bool:
+    """The reference asks Triton for its backend (dkernel/utils.py:327-331) to
+    pick tuning configurations; this build runs on ROCm only."""
+    return True
 
 
 def dense_to_crow_col(x: Tensor, include_values: bool = False) -> Tuple[Tensor, Tensor]:

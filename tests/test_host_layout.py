@@ -112,6 +112,19 @@ def test_csr_random_and_edge_cases():
                           x.numpy()[:2, :, :U.dense_to_crow_col(x)[1].max() + 1])
 
 
+def test_to_csr_matches_scipy():
+    import scipy.sparse
+    rng = np.random.default_rng(3)
+    for shape in ((1, 1), (5, 7), (16, 16), (3, 0)):
+        mat = (rng.random(shape) < 0.3) * rng.integers(1, 9, size=shape)
+        got = U.to_csr(mat)
+        want = scipy.sparse.csr_matrix(mat)
+        assert got.indptr.dtype == np.int32 and got.indices.dtype == np.int32
+        assert np.array_equal(got.indptr, want.indptr) and np.array_equal(got.indices, want.indices)
+        assert np.array_equal(got.data, want.data)
+    assert U.is_hip() is True
+
+
 def test_kv_cache_check_and_warning():
     rng = np.random.default_rng(3)
     for _ in range(20):

@@ -173,7 +173,9 @@ static int fwd_tiles_x(const FwdParams &p, int rows_per_wg) {
   const SeqView &s = p.seqs;
   int blocks;
   if (s.packed)
-    blocks = cdiv(s.max_q_len, BM) + s.batch;  // each sequence adds at most one ragged block
+    // a sequence's queries touch at most ceil(q_len / BM) + 1 row blocks (they may start inside
+    // one), and the ceilings add up to at most total / BM + batch
+    blocks = cdiv(s.max_q_len, BM) + 2 * s.batch;
   else if (s.q_starts)
     blocks = cdiv(s.max_q_len, BM) + 1;
   else {

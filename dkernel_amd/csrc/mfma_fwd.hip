@@ -750,7 +750,9 @@ int launch_mfma_fwd(const FwdParams &p, int dtype, hipStream_t stream) {
   const SeqView &s = p.seqs;
   int tiles;
   if (s.packed)
-    tiles = cdiv(s.max_q_len, 64) + s.batch;
+    // a sequence's queries touch at most ceil(q_len / 64) + 1 row blocks (they may start inside
+    // one), and the ceilings add up to at most total / 64 + batch
+    tiles = cdiv(s.max_q_len, 64) + 2 * s.batch;
   else if (s.q_starts)
     tiles = cdiv(s.max_q_len, 64) + 1;
   else {

@@ -339,6 +339,30 @@ def test_packed_varlen_prefill_and_decode(impl, D, bs):
                      atol=1e-2, rtol=1e-2)
 
 
+def test_packed_chunked_prefill_every_sequence_starts_inside_a_block(impl):
+    """Packed chunked prefill where every sequence's queries start inside a row block and end
+    in another: each touches ceil(q_len / 64) + 1 row blocks, the most the launch has to cover."""
+    Hq, Hkv, D, bs = 2, 1, 64, 64
+    sm = 1 / math.sqrt(D)
+    lens = [273, 961, 142, 434, 130, 200]
+    qlens = [252, 396, 15, 77, 66, 129]
+    g = torch.Generator().manual_seed(20)
+    ks = [torch.randn(l, Hkv, D, generator=g).to(torch.bfloat16) for l in lens]
+    vs = [torch.randn(l, Hkv, D, generator=g).to(torch.bfloat16) for l in lens]
+    qs = [torch.randn(l, Hq, D, generator=g).to(torch.bfloat16) for l in qlens]
+    cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32).to(DEV)
+    cuq = torch.tensor([0] + list(np.cumsum(qlens)), dtype=torch.int32).to(DEV)
+    mod = _module(Hq, 1024, bs, 3, 4, num_kv_heads=Hkv)
+    bm = _block_mask(Hq, 1024, bs, 3, 4, num_kv_heads=Hkv)
+    out, lse = mod(torch.cat(qs).to(DEV), torch.cat(ks).to(DEV), torch.cat(vs).to(DEV), sm,
+                   cu_seqlen_k=cu, cu_seqlen_q=cuq, return_lse=True)
+    offs = np.cumsum([0] + qlens)
+    for i in range(len(lens)):
+        ro, rl = _seq_oracle(qs[i], ks[i], vs[i], bm, bs, sm)
+        assert_close(f"O[{i}]", out[offs[i]:offs[i + 1]], ro, **TOL)
+        assert_close(f"LSE[{i}]", lse[:, offs[i]:offs[i + 1]], rl, atol=LSE_TOL, rtol=0)
+
+
 def test_c4_user_pattern_varlen_partitions(impl):
     """A reduced copy of the user-pattern configuration: per-head Bernoulli
     block pattern (diagonal forced, lower triangular), packed sequences, LSE,

@@ -15,7 +15,7 @@ import torch
 from torch import Tensor
 
 from .ops import _sparse_attention
-from .utils import (dense_to_ccol_row, get_sparse_attn_mask, is_kv_cache_efficient,
+from .utils import (dense_to_ccol_row, dense_to_crow_col, get_sparse_attn_mask, is_kv_cache_efficient,
                     masked_tile_tables, merge_split_fwd_kernel_blocks, multiple_of, split_tile_tables,
                     verify_sparse_pattern, zero_stride)
 
@@ -154,6 +154,22 @@ class SparseAttention(torch.nn.Module):
             self.register_buffer("kernel_csc_ccol", tile_csc[0].to(torch.int32), persistent=False)
             self.register_buffer("kernel_csc_row", tile_csc[1].to(torch.int32), persistent=False)
 
+        # The reference's default for blocks below 64 is a merged-row table (block_m = 64), in which
+        # a column held only by a later part of the 64 rows is attended by the earlier parts too
+        # (dkernel/utils.py:299-308): exact for local-stride patterns, not for arbitrary ones.  The
+        # layout_csr_* buffers keep that table; the kernels follow the pattern itself: unmerged
+        # tiles for the generic kernels, masked 64 x 64 tiles for the matrix-core kernels.
+        self.exact_tile = None
+        if mask_for_kernels and self.block_m != block_size:
+            exact = list(dense_to_crow_col(sparse_pattern))
+            if exact[0].dim() == 1:
+                exact = [x[None] for x in exact]
+            if exact[0].size(0) == 1:
+                exact = [zero_stride(x) for x in exact]
+            self.exact_tile = block_size
+            self.register_buffer("exact_csr_crow", exact[0].to(torch.int32), persistent=False)
+            self.register_buffer("exact_csr_col", exact[1].to(torch.int32), persistent=False)
+
         self.mask_tile = None
         if mask_for_kernels:
             m_csr, m_csc = masked_tile_tables(block_size, sparse_pattern, _KERNEL_TILE)
@@ -206,6 +222,8 @@ class SparseAttention(torch.nn.Module):
         else:
             layout_csr = (self.layout_csr_crow, self.layout_csr_col, self.block_m, self.block_n)
             layout_csc = (self.layout_csc_ccol, self.layout_csc_row, self.block_m2, self.block_n2)
+            if self.exact_tile is not None:
+                layout_csr = (self.exact_csr_crow, self.exact_csr_col, self.exact_tile, self.exact_tile)
         if self.mask_tile is not None:
             # (crow, (col, mask), tile rows, tile cols, pattern block size), longest row
             kwargs["masked_layouts"] = ((self.masked_csr_crow, self.masked_csr_col, self.mask_tile,

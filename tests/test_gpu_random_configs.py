@@ -36,14 +36,32 @@ def draw_config(rng):
     dtype = torch.bfloat16 if rng.random() < 0.7 else torch.float16
     seq_dim = int(rng.choice([1, 1, 2]))
     B = int(rng.integers(1, 4))
+    homo = bool(rng.random() < 0.15) and dense == 0 and Hkv == Hq
+    causal = bool(rng.random() < 0.85)
+    if not causal:
+        past = 0
     return dict(B=B, Hq=Hq, Hkv=Hkv, bs=bs, D=D, Lq=L, Lk=L + past, local=local, vert=vert, dense=dense,
-                dtype=dtype, seq_dim=seq_dim, dlse=bool(rng.random() < 0.3), backward=past == 0)
+                dtype=dtype, seq_dim=seq_dim, dlse=bool(rng.random() < 0.3), backward=past == 0,
+                homo=homo, offset=int(rng.integers(0, vert)), causal=causal, sliced=bool(rng.random() < 0.25))
 
 
-def run_impl(impl, mod, q, k, v, do, dlse, sm, backward):
+def to_device(x, sliced=False, seq_dim=1):
+    """Copy to the GPU; `sliced` places the data as a view inside a larger tensor (token and
+    head strides that are not the dense ones, first token not at the start)."""
+    if not sliced:
+        return x.to(DEV)
+    B, a, b, D = x.shape
+    L, H = (a, b) if seq_dim == 1 else (b, a)
+    big = torch.zeros((B, L + 8, H + 1, D) if seq_dim == 1 else (B, H + 1, L + 8, D), dtype=x.dtype, device=DEV)
+    view = big[:, 8:, :H] if seq_dim == 1 else big[:, :H, 8:]
+    view.copy_(x)
+    return view
+
+
+def run_impl(impl, mod, q, k, v, do, dlse, sm, backward, sliced=False, seq_dim=1):
     ops.set_impl(impl)
     try:
-        qd, kd, vd = (x.to(DEV).requires_grad_(backward) for x in (q, k, v))
+        qd, kd, vd = (to_device(x, sliced, seq_dim).requires_grad_(backward) for x in (q, k, v))
         out, lse = mod(qd, kd, vd, sm, return_lse=True)
         res = [out.detach().cpu(), lse.detach().cpu()]
         if backward:
@@ -76,10 +94,16 @@ def test_random_config_matches_generic_kernels_and_oracle(seed):
         kw["num_kv_heads"] = Hkv
     if c["dense"]:
         kw["num_dense_heads"] = c["dense"]
+    if c["homo"]:
+        kw["homo_head"] = True
+    if c["offset"]:
+        kw["head_sliding_offset"] = c["offset"]
+    if not c["causal"]:
+        kw["causal"] = False
     max_len = ((Lk + max(c["bs"], 64) - 1) // max(c["bs"], 64)) * max(c["bs"], 64)
     mod = LocalStrideSparseAttention(Hq, max_len, c["bs"], c["local"], c["vert"], **kw).to(DEV)
-    got = run_impl("auto", mod, q, k, v, do, dlse, sm, c["backward"])
-    ref = run_impl("generic", mod, q, k, v, do, dlse, sm, c["backward"])
+    got = run_impl("auto", mod, q, k, v, do, dlse, sm, c["backward"], c["sliced"], sd)
+    ref = run_impl("generic", mod, q, k, v, do, dlse, sm, c["backward"], c["sliced"], sd)
     names = ["O", "LSE", "dQ", "dK", "dV"]
     for name, a, b in zip(names, got, ref):
         if name == "LSE":
@@ -87,10 +111,11 @@ def test_random_config_matches_generic_kernels_and_oracle(seed):
         else:
             assert_close(f"{name} auto vs generic", a, b, **TOL)
     # oracle on the same inputs (dense fp32 attention with the token mask of the block pattern)
-    mkw = {k_: v_ for k_, v_ in kw.items() if k_ in ("num_kv_heads", "num_dense_heads")}
+    mkw = {k_: v_ for k_, v_ in kw.items() if k_ in ("num_kv_heads", "num_dense_heads", "homo_head",
+                                                      "head_sliding_offset", "causal")}
     bm = expand_heads(OL.block_mask(Hq, max_len, c["bs"], c["local"], c["vert"], **mkw), Hq)
     qo, ko, vo = (x.float().requires_grad_(c["backward"]) for x in (q, k, v))
-    ro, rl = oracle_fwd(qo, ko, vo, bm, c["bs"], sm, seq_dim=sd)
+    ro, rl = oracle_fwd(qo, ko, vo, bm, c["bs"], sm, seq_dim=sd, causal=c["causal"])
     assert_close("O vs oracle", got[0], ro, **TOL)
     assert_close("LSE vs oracle", got[1], rl, atol=LSE_TOL, rtol=0)
     if c["backward"]:

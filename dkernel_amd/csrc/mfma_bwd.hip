@@ -44,7 +44,7 @@ struct BoolConst {
 // dQ pass
 // ---------------------------------------------------------------------------
 template <typename T, int D, bool PAD, bool SUB>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void mfma_dq_kernel(const BwdParams p,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, D == 64 ? 3 : 2))) void mfma_dq_kernel(const BwdParams p,
                                                                                                    int tiles_y) {
   using M = Mma<T>;
   using vec8 = typename M::vec8;

@@ -37,8 +37,10 @@ struct FwdSmem {  // one stage = K tile + V tile, swizzled row-major (mfma_commo
   static constexpr int kStage = 2 * Tile<D>::kBytes;
 };
 
+// At the 64-wide tile a wave needs ~150 registers, so three waves fit a SIMD (three 4-wave
+// workgroups per CU): the softmax of one wave then has two others to hide behind.
 template <typename T, int D, int G, bool PAD, bool RP, bool SUB = false>
-__global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 ? 1 : 2, 2))) void mfma_fwd_kernel(const FwdParams p, int tiles_y) {
+__global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 ? 1 : 2, D == 64 ? 3 : 2))) void mfma_fwd_kernel(const FwdParams p, int tiles_y) {
   using M = Mma<T>;
   using vec8 = typename M::vec8;
   using S = FwdSmem<D>;
@@ -707,7 +709,9 @@ template <typename T, int D, bool PAD>
 static int launch_tdp(const FwdParams &p, dim3 grid, int tiles_y, hipStream_t stream) {
   static const bool row_pairs = !(getenv("DKERNEL_FWD_ROWPAIR") && atoi(getenv("DKERNEL_FWD_ROWPAIR")) == 0);
   if (row_pairs && !p.seqs.packed && fwd_group(p) == 1) return launch_row_pairs<T, D, PAD>(p, stream);
-  switch (fwd_group(p)) {
+  // 64-wide tiles: workgroups of 2 heads (4 waves), three of them per CU, beat one of 4 heads
+  const int group = D == 64 && fwd_group(p) == 4 ? 2 : fwd_group(p);
+  switch (group) {
     case 4: return launch_tdg<T, D, 4, PAD>(p, grid, tiles_y, stream);
     case 2: return launch_tdg<T, D, 2, PAD>(p, grid, tiles_y, stream);
     default: return launch_tdg<T, D, 1, PAD>(p, grid, tiles_y, stream);
@@ -728,7 +732,8 @@ static int launch_sub_g(const FwdParams &p, dim3 grid, int tiles_y, hipStream_t 
 
 template <typename T, int D>
 static int launch_sub(const FwdParams &p, dim3 grid, int tiles_y, hipStream_t stream) {
-  switch (fwd_group(p)) {
+  const int group = D == 64 && fwd_group(p) == 4 ? 2 : fwd_group(p);  // as in launch_tdp
+  switch (group) {
     case 4: return launch_sub_g<T, D, 4>(p, grid, tiles_y, stream);
     case 2: return launch_sub_g<T, D, 2>(p, grid, tiles_y, stream);
     default: return launch_sub_g<T, D, 1>(p, grid, tiles_y, stream);

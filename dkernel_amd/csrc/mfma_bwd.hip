@@ -699,7 +699,10 @@ __global__ __launch_bounds__(256) void dkdv_group_sum_kernel(const float *part_k
 // q head per kv head).
 size_t mfma_bwd_workspace_bytes(const BwdParams &p) {
   if (p.Hq == p.Hkv) return 0;
-  return 2 * (size_t)p.seqs.batch * p.Hq * p.seqs.max_k_len * p.D * sizeof(float);
+  const size_t need = 2 * (size_t)p.seqs.batch * p.Hq * p.seqs.max_k_len * p.D * sizeof(float);
+  // beyond 4 GiB of partials (large batches) the pass keeps its in-workgroup loop over the group:
+  // there are enough columns to balance then, and the scratch would rival the tensors themselves
+  return need <= ((size_t)4 << 30) ? need : 0;
 }
 
 bool mfma_bwd_supported(const BwdParams &p, int dtype) {

@@ -186,7 +186,7 @@ typedef struct dk_bwd_args {
 } dk_bwd_args;
 
 int dk_bwd(const dk_bwd_args *args);
-/* Scratch that dk_bwd can use for these arguments (0 = none useful). */
+/* Scratch that dk_bwd can use for these arguments (0 = none useful; never more than 4 GiB). */
 size_t dk_bwd_workspace_bytes(const dk_bwd_args *args);
 
 #ifdef __cplusplus

@@ -61,11 +61,31 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
   int first_rb = 0, last_rb = 0;  // RP: table rows that hold queries of this sequence
   if constexpr (RP) {
     // workgroup = table rows 2u and 2u + 1 of one head (one per wave pair); tiles_y counts pairs
-    sq = load_seq(p.seqs, blockIdx.z, p.causal);
-    if (sq.q_len <= 0) return;
-    first_rb = sq.past / 64, last_rb = (sq.past + sq.q_len - 1) / 64;
-    const int u = (first_rb >> 1) + tiles_y - 1 - (int)blockIdx.y;
-    if (u > (last_rb >> 1)) return;
+    int u;
+    if (p.seqs.packed) {
+      // the sequences share one token dimension: blockIdx.y counts row pairs over all of them
+      // (the sequences are scanned on the device, as in resolve_tile)
+      int acc = 0, found = 0;
+      for (int b = 0; b < p.seqs.batch && !found; ++b) {
+        const SeqInfo t = load_seq(p.seqs, b, p.causal);
+        if (t.q_len <= 0) continue;
+        const int f = t.past / 64, l = (t.past + t.q_len - 1) / 64;
+        const int n = (l >> 1) - (f >> 1) + 1;
+        if ((int)blockIdx.y < acc + n) {
+          sq = t, first_rb = f, last_rb = l;
+          u = (f >> 1) + (int)blockIdx.y - acc;
+          found = 1;
+        }
+        acc += n;
+      }
+      if (!found) return;
+    } else {
+      sq = load_seq(p.seqs, blockIdx.z, p.causal);
+      if (sq.q_len <= 0) return;
+      first_rb = sq.past / 64, last_rb = (sq.past + sq.q_len - 1) / 64;
+      u = (first_rb >> 1) + tiles_y - 1 - (int)blockIdx.y;
+      if (u > (last_rb >> 1)) return;
+    }
     rb = 2 * u + (wave >> 1);
     tile = rb - first_rb;  // outside [0, last_rb - first_rb]: this wave pair has no rows (row_ok false everywhere)
   } else {
@@ -667,7 +687,7 @@ static int launch_tdg(const FwdParams &p, dim3 grid, int tiles_y, hipStream_t st
   constexpr int smem = 2 * FwdSmem<D>::kStage;
   DK_ALLOW_DYNAMIC_LDS((mfma_fwd_kernel<T, D, G, PAD, false>), smem);
   grid.x = p.Hq / G;
-  // One head per workgroup (no head group to share tiles with) runs one wave per SIMD; there
+  // One head per workgroup and one q tile (row pairs switched off): one wave per SIMD, where
   // the software-pipelined kernel is the faster one.  With two waves per SIMD it is not: it
   // needs more registers than the 256 a wave gets, and spilled loader state is reloaded
   // between tile requests.  DKERNEL_FWD_PIPE=0 switches it off (A/B measurements).
@@ -683,7 +703,7 @@ static int launch_tdg(const FwdParams &p, dim3 grid, int tiles_y, hipStream_t st
   return DK_OK;
 }
 
-// One head per workgroup and every sequence in its own token dimension: two adjacent q tiles of
+// One head per workgroup: two adjacent q tiles of
 // a head share a workgroup (and the K/V tiles their rows have in common), which gives the two
 // waves per SIMD that a single 64-row tile cannot.  DKERNEL_FWD_ROWPAIR=0 switches it off.
 template <typename T, int D, bool PAD>
@@ -692,15 +712,19 @@ static int launch_row_pairs(const FwdParams &p, hipStream_t stream) {
   constexpr int smem = 2 * FwdSmem<D>::kStage;
   DK_ALLOW_DYNAMIC_LDS((mfma_fwd_kernel<T, D, 2, PAD, true>), smem);
   int pairs;
-  if (s.q_starts) {
+  if (s.packed) {
+    // per sequence at most (ceil(q_len / 64) + 1) / 2 + 1 pairs; the ceilings add up to at most
+    // total / 64 + batch
+    pairs = (cdiv(s.max_q_len, 64) + s.batch) / 2 + 2 * s.batch;
+  } else if (s.q_starts) {
     pairs = (cdiv(s.max_q_len, 64) + 1) / 2 + 1;  // a sequence's rows start anywhere inside a pair
   } else {
     const int past = p.causal ? s.max_k_len - s.max_q_len : 0;
     pairs = (((past + s.max_q_len - 1) / 64) >> 1) - ((past / 64) >> 1) + 1;
   }
   DK_REQUIRE(pairs <= 65535, "too many q tiles for one launch (%d)", pairs);
-  hipLaunchKernelGGL((mfma_fwd_kernel<T, D, 2, PAD, true>), dim3(p.Hq, pairs, s.batch), dim3(256), smem, stream, p,
-                     pairs);
+  hipLaunchKernelGGL((mfma_fwd_kernel<T, D, 2, PAD, true>), dim3(p.Hq, pairs, s.packed ? 1 : s.batch), dim3(256), smem,
+                     stream, p, pairs);
   DK_HIP_CHECK(hipGetLastError());
   return DK_OK;
 }
@@ -708,7 +732,7 @@ static int launch_row_pairs(const FwdParams &p, hipStream_t stream) {
 template <typename T, int D, bool PAD>
 static int launch_tdp(const FwdParams &p, dim3 grid, int tiles_y, hipStream_t stream) {
   static const bool row_pairs = !(getenv("DKERNEL_FWD_ROWPAIR") && atoi(getenv("DKERNEL_FWD_ROWPAIR")) == 0);
-  if (row_pairs && !p.seqs.packed && fwd_group(p) == 1) return launch_row_pairs<T, D, PAD>(p, stream);
+  if (row_pairs && fwd_group(p) == 1) return launch_row_pairs<T, D, PAD>(p, stream);
   // 64-wide tiles: workgroups of 2 heads (4 waves), three of them per CU, beat one of 4 heads
   const int group = D == 64 && fwd_group(p) == 4 ? 2 : fwd_group(p);
   switch (group) {

@@ -47,7 +47,13 @@ class SparseAttention(torch.nn.Module):
         Ignored for packed variable-length (3-D) inputs.
     block_m, block_n: kernel tile sizes on q and k (powers of 2, >= 16).
         Default block_m = max(block_size, 64) if causal else block_size,
-        block_n = block_size.
+        block_n = block_size; the attributes and the `layout_*` buffers follow
+        these defaults as in the reference.  When both are left unset and
+        block_size is not 64, the kernels themselves read extra tables built for
+        their 64 x 64 tiles (`kernel_*`: larger blocks split; `masked_*`:
+        smaller blocks as tiles with a bit mask; `exact_csr_*`: unmerged tiles
+        for the generic kernels), which follow the pattern exactly.  Explicit
+        values are honoured as given (generic kernels).
     kwargs: "out" (output tensor), "d_splits" (accepted, unused), "inference"
         (skip saving the log-sum-exp for backward; default: no input needs grad).
 

@@ -57,6 +57,11 @@ class BwdArgs(C.Structure):
                 ("workspace", vp), ("workspace_bytes", C.c_size_t), ("stream", vp)]
 
 
+class PagedKV(C.Structure):
+    _fields_ = [("block_table", vp), ("table_stride_b", i64), ("page_stride_k", i64), ("page_stride_v", i64),
+                ("page_size", i32)]
+
+
 # name -> (restype, argtypes); every symbol include/dkernel_hip.h declares
 SYMBOLS = {
     "dk_version": (C.c_int, []),
@@ -69,6 +74,7 @@ SYMBOLS = {
     "dk_kv_cache_efficient": (C.c_int, [vp, i32, i32, i32, i32, i32]),
     "dk_fwd": (C.c_int, [C.POINTER(FwdArgs)]),
     "dk_fwd_workspace_bytes": (C.c_size_t, [C.POINTER(FwdArgs)]),
+    "dk_fwd_paged": (C.c_int, [C.POINTER(FwdArgs), C.POINTER(PagedKV)]),
     "dk_bwd": (C.c_int, [C.POINTER(BwdArgs)]),
     "dk_bwd_workspace_bytes": (C.c_size_t, [C.POINTER(BwdArgs)]),
 }

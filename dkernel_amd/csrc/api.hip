@@ -96,6 +96,7 @@ static int make_fwd_params(const dk_fwd_args *a, FwdParams &p) {
   p.scale_log2 = a->sm_scale * kLog2e;
   const size_t es = elem_size(a->dtype);
   p.vec_ok = vec_aligned(a->q, es) && vec_aligned(a->k, es) && vec_aligned(a->v, es) && vec_aligned(a->o, es);
+  p.paged = PagedView{nullptr, 0, 0, 0, 0};
   return DK_OK;
 }
 
@@ -189,6 +190,30 @@ size_t dk_bwd_workspace_bytes(const dk_bwd_args *a) {
   if (make_bwd_params(a, p, empty) != DK_OK || empty) return 0;
   if (a->impl != DK_IMPL_GENERIC && mfma_bwd_supported(p, a->dtype)) return mfma_bwd_workspace_bytes(p);
   return 0;
+}
+
+int dk_fwd_paged(const dk_fwd_args *a, const dk_paged_kv *pg) {
+  clear_error();
+  DK_REQUIRE(pg != nullptr && pg->block_table != nullptr, "page table is NULL");
+  DK_REQUIRE(pg->page_size >= 16 && is_pow2(pg->page_size), "page_size must be a power of two >= 16, got %d",
+             pg->page_size);
+  FwdParams p;
+  int rc = make_fwd_params(a, p);
+  if (rc) return rc;
+  if (p.seqs.batch == 0 || p.seqs.max_q_len == 0) return DK_OK;
+  DK_REQUIRE(!p.seqs.packed && p.seqs.q_starts, "paged decode takes per-sequence lengths (dk_seqs arrays)");
+  DK_REQUIRE((pg->page_stride_k * (int64_t)elem_size(a->dtype)) % 16 == 0 &&
+                 (pg->page_stride_v * (int64_t)elem_size(a->dtype)) % 16 == 0,
+             "page strides must keep rows 16-byte aligned");
+  int shift = 0;
+  while ((1 << shift) < pg->page_size) ++shift;
+  p.paged = PagedView{pg->block_table, pg->table_stride_b, pg->page_stride_k, pg->page_stride_v, shift};
+  if (a->impl == DK_IMPL_GENERIC || !decode_supported(p, a->dtype))
+    return fail(DK_ERR_UNSUPPORTED,
+                "paged K/V is served by the split-KV decode kernels only (one query token per sequence, 16-bit "
+                "floats, head_dim a multiple of 8 up to 128, 64 x 64 tiles, causal)");
+  DK_REQUIRE(a->workspace && a->workspace_bytes >= decode_workspace_bytes(p), "decode workspace too small");
+  return launch_decode(p, a->dtype, a->workspace, a->workspace_bytes, (hipStream_t)a->stream);
 }
 
 int dk_bwd(const dk_bwd_args *a) {

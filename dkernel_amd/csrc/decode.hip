@@ -47,7 +47,7 @@ struct DecSmem {  // per wave: one 32-key half block of K and of V, plus q of th
 };
 
 // workspace layout: [batch][Hq][max_units][D + 2] floats (O[D] unnormalised, max, sum)
-template <typename T, int D, bool PAD, bool SUB>
+template <typename T, int D, bool PAD, bool SUB, bool PAGED>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void decode_partial_kernel(const FwdParams p, float *ws, int unit_blocks,
                                                             int max_units) {
   using M = Mma<T>;
@@ -82,8 +82,25 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
   const int lb = SUB ? (p.csr.sub_block == 16 ? 4 : 5) : 6, f = 64 >> lb;
   const int row_shift = ((pos & 63) >> lb) * f;
   auto half_bits = [&](int bits, int hb) { return (bits >> (row_shift + (hb & 1) * (f >> 1))) & ((1 << (f >> 1)) - 1); };
-  const T *kbase = (const T *)p.k.ptr + sq.b * p.k.sb + kvh * p.k.sh + (int64_t)sq.k_start * p.k.st;
-  const T *vbase = (const T *)p.v.ptr + sq.b * p.v.sb + kvh * p.v.sh + (int64_t)sq.k_start * p.v.st;
+  // contiguous K/V: the sequence's first key; paged K/V: the pools (pages are added per half block)
+  const T *kbase = (const T *)p.k.ptr + kvh * p.k.sh + (PAGED ? 0 : sq.b * p.k.sb + (int64_t)sq.k_start * p.k.st);
+  const T *vbase = (const T *)p.v.ptr + kvh * p.v.sh + (PAGED ? 0 : sq.b * p.v.sb + (int64_t)sq.k_start * p.v.st);
+
+  // PAGED: page numbers of the whole unit in one vector load, four lanes per table entry (a
+  // 64-key block spans at most four pages of >= 16 tokens): lane 4 j + s holds the page of keys
+  // [s, s + 1) * page_size of entry e0 + j (pages of >= 64 tokens: s = 0 only).  Entries of the
+  // page table beyond the sequence's last token are never read.
+  int my_page = 0;
+  if constexpr (PAGED) {
+    const int j = lane >> 2, s = lane & 3;
+    const int ps = 1 << p.paged.page_shift;
+    if (j < e1 - e0) {
+      const int col = cols[(e0 + j) * EW];
+      const int tok = col * 64 + (ps < 64 ? s * ps : 0);
+      if (col >= 0 && tok < sq.k_len && (s == 0 || s * ps < 64))
+        my_page = p.paged.table[b * p.paged.table_sb + (tok >> p.paged.page_shift)];
+    }
+  }
 
   // half block hb of this unit = keys cols[e0 + hb/2] * 64 + 32 * (hb & 1) + [0, 32)
   constexpr int HCH = 32 * CPR / 64;  // 16-byte chunks per lane per half tile
@@ -91,13 +108,39 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
   auto prefetch = [&](int hb, int col, int bits) {
     const int key0 = col * 64 + (hb & 1) * 32;
     if (SUB && half_bits(bits, hb) == 0) return;  // no attended key in this half: neither read nor used
+    // element offset of row r of the half block from kbase / vbase
+    int pg_lo = 0, pg_hi = 0, in_page0 = 0;
+    if constexpr (PAGED) {
+      // the half block's 32 keys lie in one page, or in two pages of 16
+      const int psl = p.paged.page_shift, half = hb & 1;
+      const int s_lo = psl < 6 ? (half * 32) >> psl : 0, s_hi = psl < 6 ? (half * 32 + 16) >> psl : 0;
+      pg_lo = __builtin_amdgcn_readlane(my_page, ((hb >> 1) * 4 + s_lo) & 63);
+      pg_hi = __builtin_amdgcn_readlane(my_page, ((hb >> 1) * 4 + s_hi) & 63);
+      in_page0 = key0 & ((1 << psl) - 1);
+    }
+    auto k_off = [&](int r) -> int64_t {
+      if constexpr (PAGED) {
+        const int in_page = (in_page0 + r) & ((1 << p.paged.page_shift) - 1);
+        return (int64_t)(r < 16 ? pg_lo : pg_hi) * p.paged.k_page_stride + (int64_t)in_page * p.k.st;
+      } else {
+        return (int64_t)(key0 + r) * p.k.st;
+      }
+    };
+    auto v_off = [&](int r) -> int64_t {
+      if constexpr (PAGED) {
+        const int in_page = (in_page0 + r) & ((1 << p.paged.page_shift) - 1);
+        return (int64_t)(r < 16 ? pg_lo : pg_hi) * p.paged.v_page_stride + (int64_t)in_page * p.v.st;
+      } else {
+        return (int64_t)(key0 + r) * p.v.st;
+      }
+    };
     if (!PAD && col >= 0 && key0 + 32 <= sq.k_len) {  // whole half inside the sequence: no guards
 #pragma unroll
       for (int c = 0; c < HCH; ++c) {
         const int idx = lane + c * 64;
         const int r = idx / CPR, ch = idx % CPR;
-        kreg[c] = *reinterpret_cast<const uint4 *>(kbase + (int64_t)(key0 + r) * p.k.st + ch * 8);
-        vreg[c] = *reinterpret_cast<const uint4 *>(vbase + (int64_t)(key0 + r) * p.v.st + ch * 8);
+        kreg[c] = *reinterpret_cast<const uint4 *>(kbase + k_off(r) + ch * 8);
+        vreg[c] = *reinterpret_cast<const uint4 *>(vbase + v_off(r) + ch * 8);
       }
     } else {  // rows beyond the sequence and (PAD) head dims beyond p.D read as zeros
 #pragma unroll
@@ -106,8 +149,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
         const int r = idx / CPR, ch = idx % CPR;
         kreg[c] = vreg[c] = make_uint4(0, 0, 0, 0);
         if (col >= 0 && key0 + r < sq.k_len && (!PAD || ch * 8 < p.D)) {
-          kreg[c] = *reinterpret_cast<const uint4 *>(kbase + (int64_t)(key0 + r) * p.k.st + ch * 8);
-          vreg[c] = *reinterpret_cast<const uint4 *>(vbase + (int64_t)(key0 + r) * p.v.st + ch * 8);
+          kreg[c] = *reinterpret_cast<const uint4 *>(kbase + k_off(r) + ch * 8);
+          vreg[c] = *reinterpret_cast<const uint4 *>(vbase + v_off(r) + ch * 8);
         }
       }
     }
@@ -336,12 +379,13 @@ size_t decode_workspace_bytes(const FwdParams &p) {
   return (size_t)p.seqs.batch * p.Hq * decode_max_units(p) * (mfma_tile_width(p.D) + 2) * sizeof(float);
 }
 
-template <typename T, int D, bool PAD, bool SUB>
+template <typename T, int D, bool PAD, bool SUB, bool PAGED>
 static int launch_decode_td(const FwdParams &p, float *ws, hipStream_t stream) {
   const int smem = DecSmem<D>::wave_bytes(p.Hq / p.Hkv);
   const int unit_blocks = decode_unit_blocks(), max_units = decode_max_units(p);
   DK_REQUIRE(max_units <= 65535, "too many decode units");
-  hipLaunchKernelGGL((decode_partial_kernel<T, D, PAD, SUB>), dim3(max_units, p.Hkv, p.seqs.batch), dim3(64), smem, stream,
+  DK_REQUIRE(!PAGED || unit_blocks <= 16, "paged decode takes at most 16 table entries per unit (DKERNEL_DECODE_UNIT)");
+  hipLaunchKernelGGL((decode_partial_kernel<T, D, PAD, SUB, PAGED>), dim3(max_units, p.Hkv, p.seqs.batch), dim3(64), smem, stream,
                      p, ws, unit_blocks, max_units);
   DK_HIP_CHECK(hipGetLastError());
   hipLaunchKernelGGL((decode_combine_kernel<T, D, PAD>), dim3(p.Hq, p.seqs.batch), dim3(64), 0, stream, p, ws,
@@ -350,16 +394,22 @@ static int launch_decode_td(const FwdParams &p, float *ws, hipStream_t stream) {
   return DK_OK;
 }
 
-// head dims below the tile width (64 or 128) run the zero-padded instantiation
+template <typename T, bool PAGED>
+static int launch_decode_tp(const FwdParams &p, float *ws, hipStream_t stream) {
+  if (p.csr.sub_block)  // entries carry a bit mask over the pattern's 16- or 32-token blocks
+    return p.D == 128 ? launch_decode_td<T, 128, false, true, PAGED>(p, ws, stream)
+                      : launch_decode_td<T, 64, false, true, PAGED>(p, ws, stream);
+  if (p.D == 128) return launch_decode_td<T, 128, false, false, PAGED>(p, ws, stream);
+  if (p.D == 64) return launch_decode_td<T, 64, false, false, PAGED>(p, ws, stream);
+  return p.D > 64 ? launch_decode_td<T, 128, true, false, PAGED>(p, ws, stream)
+                  : launch_decode_td<T, 64, true, false, PAGED>(p, ws, stream);
+}
+
+// head dims below the tile width (64 or 128) run the zero-padded instantiation; K/V come from the
+// tensors themselves or, with a page table, from page pools
 template <typename T>
 static int launch_decode_t(const FwdParams &p, float *ws, hipStream_t stream) {
-  if (p.csr.sub_block)  // entries carry a bit mask over the pattern's 16- or 32-token blocks
-    return p.D == 128 ? launch_decode_td<T, 128, false, true>(p, ws, stream)
-                      : launch_decode_td<T, 64, false, true>(p, ws, stream);
-  if (p.D == 128) return launch_decode_td<T, 128, false, false>(p, ws, stream);
-  if (p.D == 64) return launch_decode_td<T, 64, false, false>(p, ws, stream);
-  return p.D > 64 ? launch_decode_td<T, 128, true, false>(p, ws, stream)
-                  : launch_decode_td<T, 64, true, false>(p, ws, stream);
+  return p.paged.table ? launch_decode_tp<T, true>(p, ws, stream) : launch_decode_tp<T, false>(p, ws, stream);
 }
 
 int launch_decode(const FwdParams &p, int dtype, void *workspace, size_t workspace_bytes, hipStream_t stream) {

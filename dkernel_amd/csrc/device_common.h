@@ -57,11 +57,22 @@ struct SeqView {
   const int32_t *q_starts, *q_ends, *k_starts, *k_ends;
 };
 
+// Paged K/V (decode only): k / v point at page pools, token t of sequence b lives in page
+// table[b * table_sb + (t >> page_shift)] at in-page position t & (page_size - 1); inside a page
+// tokens and heads use the tensors' own token / head strides.  table == nullptr: contiguous K/V.
+struct PagedView {
+  const int32_t *table;
+  int64_t table_sb;
+  int64_t k_page_stride, v_page_stride;  // elements
+  int32_t page_shift;
+};
+
 struct FwdParams {
   TensorView q, k, v, o;
   RowView lse;
   LutView csr;
   SeqView seqs;
+  PagedView paged;
   int32_t Hq, Hkv, D, causal;
   float scale_log2;  // sm_scale * log2(e)
   int32_t vec_ok;    // 16-byte vector loads / stores are legal for q, k, v, o

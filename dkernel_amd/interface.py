@@ -244,6 +244,33 @@ class SparseAttention(torch.nn.Module):
         return output
 
 
+    def paged_decode(self, q: Tensor, k_pool: Tensor, v_pool: Tensor, block_table: Tensor,
+                     context_lens: Tensor, sm_scale: Optional[float] = None, *,
+                     return_lse: bool = False, out: Optional[Tensor] = None):
+        """One new token per sequence over a paged K/V cache (serving).
+
+        q: (batch, heads, dim) or (batch, 1, heads, dim); k_pool / v_pool: (pages, page_size,
+        kv heads, dim), page_size a power of two >= 16; block_table: int32 (batch, pages per
+        sequence); context_lens: int32 (batch,) keys per sequence including the new token's.
+        Needs the matrix-core decode kernels (bf16 / fp16, head_dim a multiple of 8 up to 128;
+        with blocks of 16 / 32: head_dim 64 or 128).  No counterpart in the reference."""
+        from .ops import paged_decode_attn
+        assert self.kwargs.get('causal', True), "paged decode is causal"
+        if self.kernel_tile is not None:
+            layout = (self.kernel_csr_crow, self.kernel_csr_col, self.kernel_tile, self.kernel_tile)
+            max_row = self.lut_max_row
+        elif self.mask_tile is not None:
+            layout = (self.masked_csr_crow, self.masked_csr_col, self.mask_tile, self.mask_tile, self.block_size)
+            max_row = self.mask_lut_max_row
+        else:
+            layout = (self.layout_csr_crow, self.layout_csr_col, self.block_m, self.block_n)
+            max_row = self.lut_max_row
+        sm_scale = sm_scale or 1. / math.sqrt(float(q.size(-1)))
+        return paged_decode_attn(q, k_pool, v_pool, block_table, context_lens, sm_scale, layout,
+                                 max_seqlen=self.max_seqlen, out=out, return_lse=return_lse,
+                                 lut_group=self.lut_group, lut_max_row=max_row)
+
+
 @lru_cache(maxsize=8)
 class LocalStrideSparseAttention(SparseAttention):
     """Local window + vertical stride pattern with per-head shifted columns

@@ -310,6 +310,58 @@ def padded_sparse_attn(q: Tensor, k: Tensor, v: Tensor, sm_scale: float,
     return (out, lse) if return_lse else out
 
 
+def paged_decode_attn(q: Tensor, k_pool: Tensor, v_pool: Tensor, block_table: Tensor, context_lens: Tensor,
+                      sm_scale: float, sparse_layout: Tuple, *, max_seqlen: int, out: Optional[Tensor] = None,
+                      return_lse: bool = False, lut_group: int = 1, lut_max_row: int = 0):
+    """One new token per sequence over a paged K/V cache.
+
+    q: (batch, heads, dim) or (batch, 1, heads, dim); k_pool, v_pool: (pages, page_size, kv heads,
+    dim) with page_size a power of two >= 16; block_table: int32 (batch, pages per sequence),
+    entry i = pool page of tokens [i, i + 1) * page_size; context_lens: int32 (batch,), keys per
+    sequence including the new token's own (the query sits at position context_len - 1).
+    Returns O shaped like q (and LSE (batch, heads, 1) when asked).  The reference has no paged
+    path (its README lists per-sequence KV-cache sizes as future work); this is the split-KV
+    decode kernel reading K/V through the page table."""
+    squeeze = q.dim() == 3
+    q4 = q[:, None] if squeeze else q
+    assert q4.dim() == 4 and q4.size(1) == 1, "paged decode takes one query token per sequence"
+    assert k_pool.dim() == 4 and k_pool.shape == v_pool.shape
+    _require_gpu(q4, k_pool, v_pool)
+    batches, num_heads, head_size = q4.size(0), q4.size(2), q4.size(3)
+    page_size, num_kv_heads = k_pool.size(1), k_pool.size(2)
+    assert k_pool.size(3) == head_size and num_heads % num_kv_heads == 0
+    assert block_table.dim() == 2 and block_table.size(0) == batches and context_lens.shape == (batches,)
+    dev = q4.device
+    q4, k_pool, v_pool = _unit_last(q4), _unit_last(k_pool), _unit_last(v_pool)
+    table = block_table.to(dev, dtype=torch.int32)
+    table = table if table.stride(1) == 1 else table.contiguous()
+    o4 = (out[:, None] if out.dim() == 3 else out) if out is not None else q4.new_empty(q4.shape)
+    lse = torch.full((batches, num_heads, 1), float("-inf"), dtype=torch.float32, device=dev) if return_lse else None
+    k_ends = context_lens.to(dev, dtype=torch.int32).contiguous()
+    zeros, ones = _const_i32(dev, batches, 0), _const_i32(dev, batches, 1)
+
+    args = _lib.FwdArgs()
+    args.q, args.o = _tensor4(q4, 2, 1), _tensor4(o4, 2, 1)
+    args.k = _lib.Tensor(k_pool.data_ptr(), 0, k_pool.stride(2), k_pool.stride(1))
+    args.v = _lib.Tensor(v_pool.data_ptr(), 0, v_pool.stride(2), v_pool.stride(1))
+    args.lse = _rowvec(lse)
+    args.csr = _lut(sparse_layout, dev, lut_group, lut_max_row)
+    capacity = min(table.size(1) * page_size, int(max_seqlen))
+    args.seqs = _lib.Seqs(batches, 1, capacity, 0, zeros.data_ptr(), ones.data_ptr(), zeros.data_ptr(), k_ends.data_ptr())
+    args.num_q_heads, args.num_kv_heads, args.head_dim = num_heads, num_kv_heads, head_size
+    args.dtype, args.causal, args.impl = _DTYPES[q4.dtype], 1, _impl
+    args.sm_scale = float(sm_scale)
+    args.stream = _stream()
+    pages = _lib.PagedKV(table.data_ptr(), table.stride(0), k_pool.stride(0), v_pool.stride(0), page_size)
+    lib = _lib.lib()
+    need = lib.dk_fwd_workspace_bytes(C.byref(args))
+    ws = torch.empty(max(need, 16), dtype=torch.uint8, device=dev)
+    args.workspace, args.workspace_bytes = ws.data_ptr(), need
+    _lib.check(lib.dk_fwd_paged(C.byref(args), C.byref(pages)))
+    res = o4[:, 0] if squeeze and out is None else (out if out is not None else o4)
+    return (res, lse) if return_lse else res
+
+
 def varlen_sparse_attn(q: Tensor, k: Tensor, v: Tensor,
                        cu_seqlens_k: Tensor, cu_seqlens_q: Optional[Tensor],
                        sm_scale: float,

@@ -160,6 +160,26 @@ int dk_fwd(const dk_fwd_args *args);
 /* Scratch that dk_fwd can use for these arguments (0 = none needed). */
 size_t dk_fwd_workspace_bytes(const dk_fwd_args *args);
 
+/* Paged K/V cache for single-token decode (serving).  args->k / args->v point at
+ * page pools: token t of sequence b lives in page block_table[b][t / page_size]
+ * at in-page position t % page_size; a page starts page_stride_k / _v elements
+ * after the previous one, tokens and heads inside a page use args->k / v
+ * stride_t / stride_h (stride_b is ignored).  page_size is a power of two >= 16.
+ * Table entries past a sequence's last token are never read.  args->seqs
+ * gives the lengths as for padded decode (q one token per sequence, k_starts 0,
+ * k_ends the context lengths, max_k_len the table's capacity in tokens) and
+ * args->workspace must hold dk_fwd_workspace_bytes(args).  No counterpart in
+ * the reference, which leaves paged caches to its callers
+ * (README.md:259-260). */
+typedef struct dk_paged_kv {
+  const int32_t *block_table; /* device, (batch, pages per sequence) */
+  int64_t table_stride_b;
+  int64_t page_stride_k, page_stride_v;
+  int32_t page_size;
+} dk_paged_kv;
+
+int dk_fwd_paged(const dk_fwd_args *args, const dk_paged_kv *pages);
+
 /* Backward of dk_fwd for equal-length, unpadded sequences (seqs pointers
  * NULL).  delta is caller scratch of batch * num_q_heads * max_q_len floats.
  * dlse.ptr may be NULL.  dk/dv are written for every kv head (sum over the q

@@ -273,6 +273,49 @@ def test_decode_head_dims_below_tile_width(impl, D, left):
     _decode_case(64, None, left, D)
 
 
+@pytest.mark.parametrize("page_size,bs,D,head_major", [(16, 64, 128, False), (32, 64, 128, True), (64, 64, 96, False),
+                                                        (128, 64, 128, False), (16, 16, 128, False),
+                                                        (32, 128, 64, True), (256, 32, 128, False)])
+def test_paged_decode(page_size, bs, D, head_major):
+    """Single-token decode over a paged K/V cache: pages scattered in the pools, table rows padded
+    with -1 past each sequence, pools token-major or head-major inside a page; against the oracle
+    on the gathered keys and against padded decode."""
+    B, Hq, Hkv, Lmax = 5, 8, 2, 2048
+    sm = 1 / math.sqrt(D)
+    g = torch.Generator().manual_seed(20)
+    lens = [64 * 21 + 12, 2048, 1, 64 * 5, 777]
+    q = torch.randn(B, Hq, D, generator=g).to(torch.bfloat16)
+    ks = [torch.randn(l, Hkv, D, generator=g).to(torch.bfloat16) for l in lens]
+    vs = [torch.randn(l, Hkv, D, generator=g).to(torch.bfloat16) for l in lens]
+    pages_per_seq = [-(-l // page_size) for l in lens]
+    num_pages = sum(pages_per_seq) + 7
+    perm = torch.randperm(num_pages, generator=g).tolist()
+    pool_shape = (num_pages, Hkv, page_size, D) if head_major else (num_pages, page_size, Hkv, D)
+    k_pool = torch.randn(pool_shape, generator=g).to(torch.bfloat16)   # stale data in unused slots
+    v_pool = torch.randn(pool_shape, generator=g).to(torch.bfloat16)
+    if head_major:
+        k_pool, v_pool = k_pool.transpose(1, 2), v_pool.transpose(1, 2)  # views: (pages, page_size, heads, dim)
+    table = torch.full((B, Lmax // page_size + 1), -1, dtype=torch.int32)
+    nxt = 0
+    for i, l in enumerate(lens):
+        for pi in range(pages_per_seq[i]):
+            pg = perm[nxt]
+            nxt += 1
+            table[i, pi] = pg
+            n = min(page_size, l - pi * page_size)
+            k_pool[pg, :n] = ks[i][pi * page_size: pi * page_size + n]
+            v_pool[pg, :n] = vs[i][pi * page_size: pi * page_size + n]
+    mod = _module(Hq, Lmax, bs, 2, 4, num_kv_heads=Hkv)
+    bm = _block_mask(Hq, Lmax, bs, 2, 4, num_kv_heads=Hkv)
+    out, lse = mod.paged_decode(q.to(DEV), k_pool.to(DEV), v_pool.to(DEV), table.to(DEV),
+                                torch.tensor(lens, dtype=torch.int32).to(DEV), sm, return_lse=True)
+    assert out.shape == (B, Hq, D) and lse.shape == (B, Hq, 1)
+    for i, l in enumerate(lens):
+        ro, rl = _seq_oracle(q[i:i + 1], ks[i], vs[i], bm, bs, sm)
+        assert_close(f"O[{i}]", out[i:i + 1], ro, **TOL)
+        assert_close(f"LSE[{i}]", lse[i], rl, atol=LSE_TOL, rtol=0)
+
+
 def _decode_case(bs, block_m, left, D):
     B, Hq, Hkv, Lmax = 4, 8, 2, 2048
     sm = 1 / math.sqrt(D)

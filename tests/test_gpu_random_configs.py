@@ -137,8 +137,8 @@ def _seq_oracle(q, k, v, bm, bs, sm):
 
 @pytest.mark.parametrize("seed", range(40))
 def test_random_inference_config_matches_generic_kernels_and_oracle(seed):
-    """Per-sequence lengths: left-padded, right-padded and packed prefill, padded and packed
-    single-token decode (split-KV kernels), chunked packed prefill."""
+    """Per-sequence lengths: left-padded, right-padded and packed prefill, padded, packed and
+    paged single-token decode (split-KV kernels), chunked packed prefill."""
     rng = np.random.default_rng(5000 + seed)
     ratio = int(rng.choice([1, 2, 4]))
     Hkv = int(rng.choice([1, 2]))
@@ -146,7 +146,10 @@ def test_random_inference_config_matches_generic_kernels_and_oracle(seed):
     bs = int(rng.choice([64, 64, 128, 16, 32]))
     D = int(rng.choice([128, 64, 96, 40]))
     dtype = torch.bfloat16 if rng.random() < 0.7 else torch.float16
-    mode = str(rng.choice(["left", "right", "packed", "packed_decode", "left_decode", "right_decode", "chunked"]))
+    mode = str(rng.choice(["left", "right", "packed", "packed_decode", "left_decode", "right_decode", "chunked",
+                           "paged_decode"]))
+    if mode == "paged_decode" and bs < 64 and D not in (64, 128):
+        D = 64  # masked tiles (blocks of 16 / 32) exist for head_dim 64 / 128 only, and paged K/V has no generic path
     nseq = int(rng.integers(1, 6))
     Lmax = int(rng.choice([256, 512, 1024]))
     lens = [int(rng.integers(1, Lmax + 1)) for _ in range(nseq)]
@@ -167,7 +170,33 @@ def test_random_inference_config_matches_generic_kernels_and_oracle(seed):
         qlens = [1 if decode else l for l in lens]
     qs = [torch.randn(ql, Hq, D, generator=g).to(dtype) for ql in qlens]
 
+    page_size = int(rng.choice([16, 32, 64, 128]))
+    page_perm = torch.randperm(sum(-(-l // page_size) for l in lens) + 3, generator=g).tolist()
+
     def call():
+        if mode == "paged_decode":
+            # pages scattered over the pools, table rows padded with -1 (never read)
+            pools = [torch.randn(len(page_perm), page_size, Hkv, D, generator=torch.Generator().manual_seed(1)).to(dtype)
+                     for _ in range(2)]
+            table = torch.full((nseq, Lmax // page_size + 1), -1, dtype=torch.int32)
+            nxt = 0
+            for i, l in enumerate(lens):
+                for pi in range(-(-l // page_size)):
+                    pg = page_perm[nxt]
+                    nxt += 1
+                    table[i, pi] = pg
+                    n = min(page_size, l - pi * page_size)
+                    pools[0][pg, :n] = ks[i][pi * page_size: pi * page_size + n]
+                    pools[1][pg, :n] = vs[i][pi * page_size: pi * page_size + n]
+            if ops._impl == ops._lib.DK_IMPL_GENERIC:
+                with pytest.raises(Exception, match="paged K/V"):
+                    mod.paged_decode(torch.cat(qs).to(DEV), pools[0].to(DEV), pools[1].to(DEV), table.to(DEV),
+                                     torch.tensor(lens, dtype=torch.int32).to(DEV), sm)
+                return None
+            out, lse = mod.paged_decode(torch.cat(qs).to(DEV), pools[0].to(DEV), pools[1].to(DEV), table.to(DEV),
+                                        torch.tensor(lens, dtype=torch.int32).to(DEV), sm, return_lse=True)
+            out, lse = out.cpu(), lse.cpu()
+            return [(out[i:i + 1], lse[i]) for i in range(nseq)]
         if mode in ("packed", "packed_decode", "chunked"):
             cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32).to(DEV)
             extra = dict(cu_seqlen_k=cu)
@@ -206,8 +235,9 @@ def test_random_inference_config_matches_generic_kernels_and_oracle(seed):
             ops.set_impl("auto")
     got, ref = with_impl("auto"), with_impl("generic")
     for i in range(nseq):
-        assert_close(f"O[{i}] auto vs generic", got[i][0], ref[i][0], **TOL)
-        assert_close(f"LSE[{i}] auto vs generic", got[i][1], ref[i][1], atol=LSE_TOL, rtol=0)
+        if ref is not None:  # (the generic kernels do not read paged caches)
+            assert_close(f"O[{i}] auto vs generic", got[i][0], ref[i][0], **TOL)
+            assert_close(f"LSE[{i}] auto vs generic", got[i][1], ref[i][1], atol=LSE_TOL, rtol=0)
         ro, rl = _seq_oracle(qs[i], ks[i], vs[i], bm, bs, sm)
         assert_close(f"O[{i}] vs oracle", got[i][0], ro, **TOL)
         assert_close(f"LSE[{i}] vs oracle", got[i][1], rl, atol=LSE_TOL, rtol=0)

@@ -12,7 +12,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 # DKERNEL_AMD_LIB points at another build of the same library (A/B comparisons of kernel variants)
 LIB_PATH = os.environ.get("DKERNEL_AMD_LIB") or os.path.join(_HERE, "libdkernel_hip.so")
 
-DK_BF16, DK_F16, DK_F32 = 0, 1, 2
+DK_BF16, DK_F16, DK_F32, DK_FP8_E4M3 = 0, 1, 2, 3
 DK_IMPL_AUTO, DK_IMPL_GENERIC, DK_IMPL_MFMA = 0, 1, 2
 DK_ERR_INVALID, DK_ERR_UNSUPPORTED, DK_ERR_HIP = -1, -2, -3
 
@@ -59,7 +59,7 @@ class BwdArgs(C.Structure):
 
 class PagedKV(C.Structure):
     _fields_ = [("block_table", vp), ("table_stride_b", i64), ("page_stride_k", i64), ("page_stride_v", i64),
-                ("page_size", i32)]
+                ("page_size", i32), ("kv_dtype", i32), ("k_scale", f32), ("v_scale", f32)]
 
 
 # name -> (restype, argtypes); every symbol include/dkernel_hip.h declares

@@ -202,12 +202,22 @@ int dk_fwd_paged(const dk_fwd_args *a, const dk_paged_kv *pg) {
   if (rc) return rc;
   if (p.seqs.batch == 0 || p.seqs.max_q_len == 0) return DK_OK;
   DK_REQUIRE(!p.seqs.packed && p.seqs.q_starts, "paged decode takes per-sequence lengths (dk_seqs arrays)");
-  DK_REQUIRE((pg->page_stride_k * (int64_t)elem_size(a->dtype)) % 16 == 0 &&
-                 (pg->page_stride_v * (int64_t)elem_size(a->dtype)) % 16 == 0,
+  DK_REQUIRE(pg->kv_dtype == DK_FP8_E4M3 || ((pg->page_stride_k * (int64_t)elem_size(a->dtype)) % 16 == 0 &&
+                                              (pg->page_stride_v * (int64_t)elem_size(a->dtype)) % 16 == 0),
              "page strides must keep rows 16-byte aligned");
   int shift = 0;
   while ((1 << shift) < pg->page_size) ++shift;
-  p.paged = PagedView{pg->block_table, pg->table_stride_b, pg->page_stride_k, pg->page_stride_v, shift};
+  const bool fp8 = pg->kv_dtype == DK_FP8_E4M3;
+  DK_REQUIRE(fp8 || pg->kv_dtype == a->dtype, "kv_dtype must be the q dtype or DK_FP8_E4M3, got %d", pg->kv_dtype);
+  DK_REQUIRE(!fp8 || (pg->k_scale > 0.f && pg->v_scale > 0.f), "fp8 K/V scales must be positive");
+  const int64_t kv_es = fp8 ? 1 : (int64_t)elem_size(a->dtype);
+  DK_REQUIRE((pg->page_stride_k * kv_es) % 8 == 0 && (pg->page_stride_v * kv_es) % 8 == 0 &&
+                 (!fp8 || (a->k.stride_h % 8 == 0 && a->k.stride_t % 8 == 0 && a->v.stride_h % 8 == 0 &&
+                           a->v.stride_t % 8 == 0 && ((uintptr_t)a->k.ptr % 8) == 0 && ((uintptr_t)a->v.ptr % 8) == 0)),
+             "fp8 K/V rows must be 8-byte aligned");
+  p.paged = PagedView{pg->block_table, pg->table_stride_b, pg->page_stride_k, pg->page_stride_v, shift,
+                      fp8 ? 1 : 0, fp8 ? pg->v_scale : 1.f};
+  if (fp8) p.scale_log2 *= pg->k_scale;  // S = (q . k8) k_scale sm_scale
   if (a->impl == DK_IMPL_GENERIC || !decode_supported(p, a->dtype))
     return fail(DK_ERR_UNSUPPORTED,
                 "paged K/V is served by the split-KV decode kernels only (one query token per sequence, 16-bit "

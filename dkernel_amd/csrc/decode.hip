@@ -21,6 +21,7 @@
 // CU (2 per SIMD, <= 256 VGPRs each): one wave's loads overlap the other's
 // multiplies on the same SIMD.
 #include <cstdlib>
+#include <type_traits>
 
 #include "common.h"
 #include "device_common.h"
@@ -47,7 +48,30 @@ struct DecSmem {  // per wave: one 32-key half block of K and of V, plus q of th
 };
 
 // workspace layout: [batch][Hq][max_units][D + 2] floats (O[D] unnormalised, max, sum)
-template <typename T, int D, bool PAD, bool SUB, bool PAGED>
+// Eight OCP e4m3 bytes -> eight elements of T.  Exact (e4m3 has 3 mantissa bits), so bf16 is
+// the upper half of the fp32 value and fp16 needs no rounding mode: one convert and one pack per
+// two elements.
+template <typename T>
+__device__ __forceinline__ uint32_t pack2_exact(float a, float b);
+template <>
+__device__ __forceinline__ uint32_t pack2_exact<bf16_t>(float a, float b) {
+  return __builtin_amdgcn_perm(__float_as_uint(b), __float_as_uint(a), 0x07060302u);  // hi16(b) : hi16(a)
+}
+template <>
+__device__ __forceinline__ uint32_t pack2_exact<f16_t>(float a, float b) {
+  return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(a, b));
+}
+template <typename T>
+__device__ __forceinline__ uint4 fp8x8_to(uint2 w) {
+  typedef float float2_ __attribute__((ext_vector_type(2)));
+  const float2_ a = __builtin_amdgcn_cvt_pk_f32_fp8((int)w.x, false), b = __builtin_amdgcn_cvt_pk_f32_fp8((int)w.x, true);
+  const float2_ c = __builtin_amdgcn_cvt_pk_f32_fp8((int)w.y, false), d = __builtin_amdgcn_cvt_pk_f32_fp8((int)w.y, true);
+  return make_uint4(pack2_exact<T>(a[0], a[1]), pack2_exact<T>(b[0], b[1]), pack2_exact<T>(c[0], c[1]),
+                    pack2_exact<T>(d[0], d[1]));
+}
+
+// KV8 (with PAGED): the K/V pools hold fp8 bytes, converted to T on the way into LDS.
+template <typename T, int D, bool PAD, bool SUB, bool PAGED, bool KV8 = false>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void decode_partial_kernel(const FwdParams p, float *ws, int unit_blocks,
                                                             int max_units) {
   using M = Mma<T>;
@@ -83,8 +107,16 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
   const int row_shift = ((pos & 63) >> lb) * f;
   auto half_bits = [&](int bits, int hb) { return (bits >> (row_shift + (hb & 1) * (f >> 1))) & ((1 << (f >> 1)) - 1); };
   // contiguous K/V: the sequence's first key; paged K/V: the pools (pages are added per half block)
-  const T *kbase = (const T *)p.k.ptr + kvh * p.k.sh + (PAGED ? 0 : sq.b * p.k.sb + (int64_t)sq.k_start * p.k.st);
-  const T *vbase = (const T *)p.v.ptr + kvh * p.v.sh + (PAGED ? 0 : sq.b * p.v.sb + (int64_t)sq.k_start * p.v.st);
+  static_assert(!KV8 || PAGED, "fp8 K/V comes through the paged entry");
+  using KV = typename std::conditional<KV8, uint8_t, T>::type;  // element type of the K/V memory
+  const KV *kbase = (const KV *)p.k.ptr + kvh * p.k.sh + (PAGED ? 0 : sq.b * p.k.sb + (int64_t)sq.k_start * p.k.st);
+  const KV *vbase = (const KV *)p.v.ptr + kvh * p.v.sh + (PAGED ? 0 : sq.b * p.v.sb + (int64_t)sq.k_start * p.v.st);
+  auto load8 = [](const KV *src) -> uint4 {  // 8 head dims starting at src, as T
+    if constexpr (KV8)
+      return fp8x8_to<T>(*reinterpret_cast<const uint2 *>(src));
+    else
+      return *reinterpret_cast<const uint4 *>(src);
+  };
 
   // PAGED: page numbers of the whole unit in one vector load, four lanes per table entry (a
   // 64-key block spans at most four pages of >= 16 tokens): lane 4 j + s holds the page of keys
@@ -139,8 +171,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
       for (int c = 0; c < HCH; ++c) {
         const int idx = lane + c * 64;
         const int r = idx / CPR, ch = idx % CPR;
-        kreg[c] = *reinterpret_cast<const uint4 *>(kbase + k_off(r) + ch * 8);
-        vreg[c] = *reinterpret_cast<const uint4 *>(vbase + v_off(r) + ch * 8);
+        kreg[c] = load8(kbase + k_off(r) + ch * 8);
+        vreg[c] = load8(vbase + v_off(r) + ch * 8);
       }
     } else {  // rows beyond the sequence and (PAD) head dims beyond p.D read as zeros
 #pragma unroll
@@ -149,8 +181,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
         const int r = idx / CPR, ch = idx % CPR;
         kreg[c] = vreg[c] = make_uint4(0, 0, 0, 0);
         if (col >= 0 && key0 + r < sq.k_len && (!PAD || ch * 8 < p.D)) {
-          kreg[c] = *reinterpret_cast<const uint4 *>(kbase + k_off(r) + ch * 8);
-          vreg[c] = *reinterpret_cast<const uint4 *>(vbase + v_off(r) + ch * 8);
+          kreg[c] = load8(kbase + k_off(r) + ch * 8);
+          vreg[c] = load8(vbase + v_off(r) + ch * 8);
         }
       }
     }
@@ -348,11 +380,11 @@ __global__ __launch_bounds__(64) void decode_combine_kernel(const FwdParams p, c
     }
     mmax = mnew;
   }
-  const float inv = l > 0.f ? 1.f / l : 0.f;
+  const float inv = l > 0.f ? (p.paged.table ? p.paged.out_scale : 1.f) / l : 0.f;
   T *op = (T *)p.o.ptr + sq.b * p.o.sb + h * p.o.sh + (int64_t)sq.q_start * p.o.st;
 #pragma unroll
   for (int i = 0; i < PER; ++i)
-    if (!PAD || lane * PER + i < p.D) op[lane * PER + i] = from_float<T>(o[i] * inv);
+    if (!PAD || lane * PER + i < p.D) op[lane * PER + i] = from_float<T>(o[i] * inv);  // inv includes the V scale
   if (p.lse.ptr && lane == 0)
     p.lse.ptr[sq.b * p.lse.sb + h * p.lse.sh + (int64_t)sq.q_start * p.lse.st] =
         l > 0.f ? (mmax + log2f(l)) * kLn2 : -INFINITY;
@@ -379,13 +411,13 @@ size_t decode_workspace_bytes(const FwdParams &p) {
   return (size_t)p.seqs.batch * p.Hq * decode_max_units(p) * (mfma_tile_width(p.D) + 2) * sizeof(float);
 }
 
-template <typename T, int D, bool PAD, bool SUB, bool PAGED>
+template <typename T, int D, bool PAD, bool SUB, bool PAGED, bool KV8 = false>
 static int launch_decode_td(const FwdParams &p, float *ws, hipStream_t stream) {
   const int smem = DecSmem<D>::wave_bytes(p.Hq / p.Hkv);
   const int unit_blocks = decode_unit_blocks(), max_units = decode_max_units(p);
   DK_REQUIRE(max_units <= 65535, "too many decode units");
   DK_REQUIRE(!PAGED || unit_blocks <= 16, "paged decode takes at most 16 table entries per unit (DKERNEL_DECODE_UNIT)");
-  hipLaunchKernelGGL((decode_partial_kernel<T, D, PAD, SUB, PAGED>), dim3(max_units, p.Hkv, p.seqs.batch), dim3(64), smem, stream,
+  hipLaunchKernelGGL((decode_partial_kernel<T, D, PAD, SUB, PAGED, KV8>), dim3(max_units, p.Hkv, p.seqs.batch), dim3(64), smem, stream,
                      p, ws, unit_blocks, max_units);
   DK_HIP_CHECK(hipGetLastError());
   hipLaunchKernelGGL((decode_combine_kernel<T, D, PAD>), dim3(p.Hq, p.seqs.batch), dim3(64), 0, stream, p, ws,
@@ -409,6 +441,12 @@ static int launch_decode_tp(const FwdParams &p, float *ws, hipStream_t stream) {
 // tensors themselves or, with a page table, from page pools
 template <typename T>
 static int launch_decode_t(const FwdParams &p, float *ws, hipStream_t stream) {
+  if (p.paged.table && p.paged.kv_fp8) {  // fp8 pools: plain tiles only
+    if (p.csr.sub_block || (p.D != 64 && p.D != 128))
+      return fail(DK_ERR_UNSUPPORTED, "fp8 K/V needs head_dim 64 or 128 and pattern blocks of at least 64");
+    return p.D == 128 ? launch_decode_td<T, 128, false, false, true, true>(p, ws, stream)
+                      : launch_decode_td<T, 64, false, false, true, true>(p, ws, stream);
+  }
   return p.paged.table ? launch_decode_tp<T, true>(p, ws, stream) : launch_decode_tp<T, false>(p, ws, stream);
 }
 

@@ -65,6 +65,8 @@ struct PagedView {
   int64_t table_sb;
   int64_t k_page_stride, v_page_stride;  // elements
   int32_t page_shift;
+  int32_t kv_fp8;    // pools hold OCP e4m3 bytes (k / v strides then count bytes); q / o keep their type
+  float out_scale;   // V scale of an fp8 cache, applied to O (the K scale is folded into scale_log2)
 };
 
 struct FwdParams {

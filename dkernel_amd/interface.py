@@ -246,13 +246,15 @@ class SparseAttention(torch.nn.Module):
 
     def paged_decode(self, q: Tensor, k_pool: Tensor, v_pool: Tensor, block_table: Tensor,
                      context_lens: Tensor, sm_scale: Optional[float] = None, *,
-                     return_lse: bool = False, out: Optional[Tensor] = None):
+                     return_lse: bool = False, out: Optional[Tensor] = None,
+                     k_scale: float = 1.0, v_scale: float = 1.0):
         """One new token per sequence over a paged K/V cache (serving).
 
         q: (batch, heads, dim) or (batch, 1, heads, dim); k_pool / v_pool: (pages, page_size,
         kv heads, dim), page_size a power of two >= 16; block_table: int32 (batch, pages per
         sequence); context_lens: int32 (batch,) keys per sequence including the new token's.
-        Needs the matrix-core decode kernels (bf16 / fp16, head_dim a multiple of 8 up to 128;
+        Pools of dtype torch.float8_e4m3fn hold K / k_scale and V / v_scale (head_dim 64 / 128,
+        blocks of at least 64).  Needs the matrix-core decode kernels (bf16 / fp16, head_dim a multiple of 8 up to 128;
         with blocks of 16 / 32: head_dim 64 or 128).  No counterpart in the reference."""
         from .ops import paged_decode_attn
         assert self.kwargs.get('causal', True), "paged decode is causal"
@@ -268,7 +270,8 @@ class SparseAttention(torch.nn.Module):
         sm_scale = sm_scale or 1. / math.sqrt(float(q.size(-1)))
         return paged_decode_attn(q, k_pool, v_pool, block_table, context_lens, sm_scale, layout,
                                  max_seqlen=self.max_seqlen, out=out, return_lse=return_lse,
-                                 lut_group=self.lut_group, lut_max_row=max_row)
+                                 lut_group=self.lut_group, lut_max_row=max_row,
+                                 k_scale=k_scale, v_scale=v_scale)
 
 
 @lru_cache(maxsize=8)

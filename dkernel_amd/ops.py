@@ -312,13 +312,16 @@ def padded_sparse_attn(q: Tensor, k: Tensor, v: Tensor, sm_scale: float,
 
 def paged_decode_attn(q: Tensor, k_pool: Tensor, v_pool: Tensor, block_table: Tensor, context_lens: Tensor,
                       sm_scale: float, sparse_layout: Tuple, *, max_seqlen: int, out: Optional[Tensor] = None,
-                      return_lse: bool = False, lut_group: int = 1, lut_max_row: int = 0):
+                      return_lse: bool = False, lut_group: int = 1, lut_max_row: int = 0,
+                      k_scale: float = 1.0, v_scale: float = 1.0):
     """One new token per sequence over a paged K/V cache.
 
     q: (batch, heads, dim) or (batch, 1, heads, dim); k_pool, v_pool: (pages, page_size, kv heads,
     dim) with page_size a power of two >= 16; block_table: int32 (batch, pages per sequence),
     entry i = pool page of tokens [i, i + 1) * page_size; context_lens: int32 (batch,), keys per
     sequence including the new token's own (the query sits at position context_len - 1).
+    Pools of dtype torch.float8_e4m3fn hold K / k_scale and V / v_scale (per-tensor scales; head_dim
+    64 or 128, pattern blocks of at least 64); otherwise the pools have q's dtype.
     Returns O shaped like q (and LSE (batch, heads, 1) when asked).  The reference has no paged
     path (its README lists per-sequence KV-cache sizes as future work); this is the split-KV
     decode kernel reading K/V through the page table."""
@@ -326,7 +329,8 @@ def paged_decode_attn(q: Tensor, k_pool: Tensor, v_pool: Tensor, block_table: Te
     q4 = q[:, None] if squeeze else q
     assert q4.dim() == 4 and q4.size(1) == 1, "paged decode takes one query token per sequence"
     assert k_pool.dim() == 4 and k_pool.shape == v_pool.shape
-    _require_gpu(q4, k_pool, v_pool)
+    _require_gpu(q4)
+    assert k_pool.is_cuda and v_pool.is_cuda and k_pool.dtype == v_pool.dtype
     batches, num_heads, head_size = q4.size(0), q4.size(2), q4.size(3)
     page_size, num_kv_heads = k_pool.size(1), k_pool.size(2)
     assert k_pool.size(3) == head_size and num_heads % num_kv_heads == 0
@@ -352,7 +356,10 @@ def paged_decode_attn(q: Tensor, k_pool: Tensor, v_pool: Tensor, block_table: Te
     args.dtype, args.causal, args.impl = _DTYPES[q4.dtype], 1, _impl
     args.sm_scale = float(sm_scale)
     args.stream = _stream()
-    pages = _lib.PagedKV(table.data_ptr(), table.stride(0), k_pool.stride(0), v_pool.stride(0), page_size)
+    fp8 = k_pool.dtype == torch.float8_e4m3fn
+    assert fp8 or k_pool.dtype == q4.dtype, f"K/V pools must have q's dtype or float8_e4m3fn, got {k_pool.dtype}"
+    pages = _lib.PagedKV(table.data_ptr(), table.stride(0), k_pool.stride(0), v_pool.stride(0), page_size,
+                         _lib.DK_FP8_E4M3 if fp8 else _DTYPES[q4.dtype], float(k_scale), float(v_scale))
     lib = _lib.lib()
     need = lib.dk_fwd_workspace_bytes(C.byref(args))
     ws = torch.empty(max(need, 16), dtype=torch.uint8, device=dev)

@@ -25,7 +25,8 @@ extern "C" {
 #define DK_ERR_UNSUPPORTED (-2) /* shape / dtype without a kernel */
 #define DK_ERR_HIP (-3)         /* a HIP runtime call failed */
 
-enum dk_dtype { DK_BF16 = 0, DK_F16 = 1, DK_F32 = 2 };
+enum dk_dtype { DK_BF16 = 0, DK_F16 = 1, DK_F32 = 2,
+                DK_FP8_E4M3 = 3 /* OCP e4m3 bytes; K/V pools of dk_fwd_paged only */ };
 enum dk_impl { DK_IMPL_AUTO = 0, DK_IMPL_GENERIC = 1, DK_IMPL_MFMA = 2 };
 
 int dk_version(void);              /* 10000*major + 100*minor + patch */
@@ -169,13 +170,17 @@ size_t dk_fwd_workspace_bytes(const dk_fwd_args *args);
  * gives the lengths as for padded decode (q one token per sequence, k_starts 0,
  * k_ends the context lengths, max_k_len the table's capacity in tokens) and
  * args->workspace must hold dk_fwd_workspace_bytes(args).  No counterpart in
- * the reference, which leaves paged caches to its callers
- * (README.md:259-260). */
+ * the reference, which lists per-sequence cache sizes and FP8 as future work
+ * (README.md:257-260). */
 typedef struct dk_paged_kv {
   const int32_t *block_table; /* device, (batch, pages per sequence) */
   int64_t table_stride_b;
   int64_t page_stride_k, page_stride_v;
   int32_t page_size;
+  int32_t kv_dtype;     /* args->dtype (pools hold q's type), or DK_FP8_E4M3: the pools hold bytes,
+                           value = byte as e4m3 * k_scale / v_scale, and all K/V strides count
+                           bytes; head_dim 64 or 128, pattern blocks >= 64 */
+  float k_scale, v_scale; /* used with DK_FP8_E4M3 */
 } dk_paged_kv;
 
 int dk_fwd_paged(const dk_fwd_args *args, const dk_paged_kv *pages);

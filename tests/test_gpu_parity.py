@@ -316,6 +316,47 @@ def test_paged_decode(page_size, bs, D, head_major):
         assert_close(f"LSE[{i}]", lse[i], rl, atol=LSE_TOL, rtol=0)
 
 
+@pytest.mark.parametrize("page_size,bs,D,dtype", [(16, 64, 128, torch.bfloat16), (64, 128, 64, torch.float16)])
+def test_paged_decode_fp8_cache(page_size, bs, D, dtype):
+    """Paged decode over OCP e4m3 K/V pools with per-tensor scales: the oracle attends to the
+    dequantised keys and values (byte as e4m3 times the scale), which the kernel reproduces
+    exactly before its 16-bit products."""
+    B, Hq, Hkv, Lmax = 4, 8, 2, 1024
+    sm = 1 / math.sqrt(D)
+    g = torch.Generator().manual_seed(20)
+    lens = [1000, 65, 1, 513]
+    k_scale, v_scale = 0.05, 0.125
+    q = torch.randn(B, Hq, D, generator=g).to(dtype)
+    ks8 = [(torch.randn(l, Hkv, D, generator=g) / k_scale).to(torch.float8_e4m3fn) for l in lens]
+    vs8 = [(torch.randn(l, Hkv, D, generator=g) / v_scale).to(torch.float8_e4m3fn) for l in lens]
+    pages_per_seq = [-(-l // page_size) for l in lens]
+    num_pages = sum(pages_per_seq) + 3
+    perm = torch.randperm(num_pages, generator=g).tolist()
+    k_pool = torch.zeros(num_pages, page_size, Hkv, D, dtype=torch.uint8)
+    v_pool = torch.zeros_like(k_pool)
+    table = torch.full((B, Lmax // page_size), -1, dtype=torch.int32)
+    nxt = 0
+    for i, l in enumerate(lens):
+        for pi in range(pages_per_seq[i]):
+            pg = perm[nxt]
+            nxt += 1
+            table[i, pi] = pg
+            n = min(page_size, l - pi * page_size)
+            k_pool[pg, :n] = ks8[i][pi * page_size: pi * page_size + n].view(torch.uint8)
+            v_pool[pg, :n] = vs8[i][pi * page_size: pi * page_size + n].view(torch.uint8)
+    mod = _module(Hq, Lmax, bs, 2, 4, num_kv_heads=Hkv)
+    bm = _block_mask(Hq, Lmax, bs, 2, 4, num_kv_heads=Hkv)
+    out, lse = mod.paged_decode(q.to(DEV), k_pool.to(DEV).view(torch.float8_e4m3fn),
+                                v_pool.to(DEV).view(torch.float8_e4m3fn), table.to(DEV),
+                                torch.tensor(lens, dtype=torch.int32).to(DEV), sm, return_lse=True,
+                                k_scale=k_scale, v_scale=v_scale)
+    for i, l in enumerate(lens):
+        kd, vd = ks8[i].float() * k_scale, vs8[i].float() * v_scale
+        ro, rl = _seq_oracle(q[i:i + 1].float(), kd, vd, bm, bs, sm)
+        assert_close(f"O[{i}]", out[i:i + 1], ro, **TOL)
+        assert_close(f"LSE[{i}]", lse[i], rl, atol=LSE_TOL, rtol=0)
+
+
 def _decode_case(bs, block_m, left, D):
     B, Hq, Hkv, Lmax = 4, 8, 2, 2048
     sm = 1 / math.sqrt(D)

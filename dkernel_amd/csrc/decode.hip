@@ -20,6 +20,7 @@
 // the next half block prefetched into registers, so 8 waves are resident per
 // CU (2 per SIMD, <= 256 VGPRs each): one wave's loads overlap the other's
 // multiplies on the same SIMD.
+#include <algorithm>
 #include <cstdlib>
 #include <type_traits>
 
@@ -29,14 +30,36 @@
 
 namespace dk {
 
-// Blocks per work unit (one wave).  Equal-sized units keep every wave busy for
-// the same time whatever the KV lengths are; 6 blocks = 192 KB per unit.
-static int decode_unit_blocks() {
+constexpr int kDecodeWaves = 4;  // units (waves) per workgroup
+
+// Upper bound on the entries of one table row: the caller's hint when given,
+// else the number of column blocks.
+static int decode_max_row_entries(const FwdParams &p) {
+  return p.csr.max_row_entries > 0 ? p.csr.max_row_entries : p.csr.num_rows;
+}
+
+// Table entries per work unit (one wave).  With enough rows (sequences x kv heads) to fill the
+// machine, a row is cut into as many units as a workgroup has waves, so that it is finished
+// inside one workgroup and the merge kernel is not launched at all; with few rows, into more
+// units (about 1024 waves in total).  At most 16 (the paged path keeps a unit's page numbers in
+// the lanes of one register).  DKERNEL_DECODE_UNIT overrides.
+static int decode_unit_blocks(const FwdParams &p) {
   if (const char *env = getenv("DKERNEL_DECODE_UNIT")) {
     const int v = atoi(env);
-    if (v >= 1 && v <= 64) return v;
+    if (v >= 1 && v <= 16) return v;
   }
-  return 6;
+  const int rows = p.seqs.batch * p.Hkv;
+  const int units_per_row = std::max(kDecodeWaves, cdiv(1024, rows > 0 ? rows : 1));
+  return std::min(16, std::max(2, cdiv(decode_max_row_entries(p), units_per_row)));
+}
+
+// Units a row of n table entries is cut into: as many as the unit size asks for, and at least
+// the waves of one workgroup (one entry each at worst), so that every wave of the workgroup that
+// finishes a row streams a share of it.  Used by both kernels.
+__host__ __device__ inline int decode_row_units(int n, int unit_blocks, int waves) {
+  const int by_size = (n + unit_blocks - 1) / unit_blocks;
+  const int by_waves = n < waves ? n : waves;
+  return by_size > by_waves ? by_size : by_waves;
 }
 
 template <int D>
@@ -71,9 +94,12 @@ __device__ __forceinline__ uint4 fp8x8_to(uint2 w) {
 }
 
 // KV8 (with PAGED): the K/V pools hold fp8 bytes, converted to T on the way into LDS.
-template <typename T, int D, bool PAD, bool SUB, bool PAGED, bool KV8 = false>
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void decode_partial_kernel(const FwdParams p, float *ws, int unit_blocks,
-                                                            int max_units) {
+// W waves per workgroup = W consecutive units of one row.  A row whose units all sit in one
+// workgroup is finished here (the waves exchange their partials through LDS and write O / LSE);
+// longer rows leave their partials in the workspace for decode_combine_kernel.
+template <typename T, int D, bool PAD, bool SUB, bool PAGED, bool KV8, int W>
+__global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(2, 2))) void decode_partial_kernel(
+    const FwdParams p, float *ws, int unit_blocks, int max_units) {
   using M = Mma<T>;
   using vec8 = typename M::vec8;
   using S = DecSmem<D>;
@@ -81,25 +107,35 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
   // SUB: table entries are (column, bit mask over the pattern blocks inside the 64 x 64 tile)
   static_assert(!SUB || !PAD, "sub-block masks: plain tiles only");
   constexpr int EW = SUB ? 2 : 1;  // ints per table entry
-  extern __shared__ __align__(16) char smem[];
+  extern __shared__ __align__(16) char smem_all[];
 
-  const int unit = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+  const int kvh = blockIdx.y, b = blockIdx.z;
   const SeqInfo sq = load_seq(p.seqs, b, p.causal);
-  if (sq.q_len <= 0 || sq.k_len <= 0) return;
+  if (sq.q_len <= 0) return;
   const int ratio = __builtin_amdgcn_readfirstlane(p.Hq / p.Hkv);  // integer division runs on the VALU
-  const int lane = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int wave_bytes = 2 * S::kHalf + ratio * D * 2;
+  char *smem = smem_all + wave * wave_bytes;  // this wave's private tiles and q copy
   const int m = lane & 31, g = lane >> 5;  // m = q head inside the group (MFMA column)
   const int pos = sq.past;                 // absolute position of the single query token
   const int rb = pos / 64;
   const int h0 = kvh * ratio;
   const int lh = lut_head(p.csr, h0, p.Hq, p.Hkv);
-  if (rb >= p.csr.num_rows) return;
   // table reads go through the scalar unit (wave-uniform addresses, no vector-memory wait)
-  int row0, row1;
-  scalar_load2(p.csr.ptr + lh * p.csr.ptr_sh + rb, p.csr.ptr + lh * p.csr.ptr_sh + rb + 1, row0, row1);
-  const int e0 = row0 + unit * unit_blocks;
-  if (e0 >= row1) return;  // this row has fewer units
-  const int e1 = min(e0 + unit_blocks, row1);
+  int row0 = 0, row1 = 0;
+  if (sq.k_len > 0 && rb < p.csr.num_rows)
+    scalar_load2(p.csr.ptr + lh * p.csr.ptr_sh + rb, p.csr.ptr + lh * p.csr.ptr_sh + rb + 1, row0, row1);
+  // the row's entries are split evenly over as many units as the unit size asks for
+  const int n_ent = row1 - row0;
+  const int u_cnt = decode_row_units(n_ent, unit_blocks, W);
+  if ((int)blockIdx.x * W >= u_cnt && (blockIdx.x > 0 || W == 1)) return;  // nothing for this workgroup
+  const bool merge_here = W > 1 && u_cnt <= W;  // (a row without entries is written here too: O = 0, LSE = -inf)
+  const int per = u_cnt > 0 ? (n_ent + u_cnt - 1) / u_cnt : 0;
+  const int unit = blockIdx.x * W + wave;
+  const bool active = unit < u_cnt;
+  if (!active && !merge_here) return;
+  const int e0 = row0 + unit * per;
+  const int e1 = active ? min(e0 + per, row1) : e0;
   const int32_t *cols = p.csr.idx + lh * p.csr.idx_sh;
   // SUB: the query's row of pattern blocks inside its tile selects f of the entry's f x f mask
   // bits; half block hb & 1 holds key parts [hb & 1, hb & 1 + 1) * f / 2 of them
@@ -188,12 +224,14 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
     }
   };
   // the first K/V request goes out before anything else touches memory
-  int col_cur, bits_cur = 0;
-  if constexpr (SUB)
-    scalar_load2(cols + e0 * EW, cols + e0 * EW + 1, col_cur, bits_cur);
-  else
-    col_cur = scalar_load(cols + e0);
-  prefetch(0, col_cur, bits_cur);
+  int col_cur = 0, bits_cur = 0;
+  if (active) {
+    if constexpr (SUB)
+      scalar_load2(cols + e0 * EW, cols + e0 * EW + 1, col_cur, bits_cur);
+    else
+      col_cur = scalar_load(cols + e0);
+    prefetch(0, col_cur, bits_cur);
+  }
 
   // q of the group's heads -> LDS (row min(m, ratio-1) feeds MFMA column m;
   // columns >= ratio are duplicates whose results are never stored)
@@ -314,8 +352,11 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
   }
 
   // ---- partial result of this unit: lanes (m < ratio) hold head h0 + m ----
+  // rows [head][D + 2] floats (O unnormalised, max, sum): in the workspace, or, when the row is
+  // finished here, in this wave's own tile area (its tiles are dead by now)
   if (m < ratio) {
-    float *dst = ws + (((int64_t)b * p.Hq + h0 + m) * max_units + unit) * (D + 2);
+    float *dst = merge_here ? reinterpret_cast<float *>(smem) + m * (D + 2)
+                            : ws + (((int64_t)b * p.Hq + h0 + m) * max_units + unit) * (D + 2);
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -327,6 +368,45 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
       dst[D + 1] = l_run;
     }
   }
+  if constexpr (W > 1) {
+    if (!merge_here) return;
+    __syncthreads();  // every wave of the workgroup gets here (merge_here is workgroup-uniform)
+    // heads of the group are dealt to the waves; lane l owns dims l D/64 .. of its head
+    constexpr int PER = D / 64;
+    for (int h = wave; h < ratio; h += W) {
+      float mv[W], lv[W], ov[W][PER];
+#pragma unroll
+      for (int u = 0; u < W; ++u) {
+        const float *row = reinterpret_cast<const float *>(smem_all + u * wave_bytes) + h * (D + 2);
+        mv[u] = row[D];
+        lv[u] = row[D + 1];
+#pragma unroll
+        for (int i = 0; i < PER; ++i) ov[u][i] = row[lane * PER + i];
+      }
+      float mmax = mv[0];
+#pragma unroll
+      for (int u = 1; u < W; ++u) mmax = fmaxf(mmax, mv[u]);
+      const float muse = mmax == -INFINITY ? 0.f : mmax;
+      float l = 0.f, o[PER];
+#pragma unroll
+      for (int i = 0; i < PER; ++i) o[i] = 0.f;
+#pragma unroll
+      for (int u = 0; u < W; ++u) {
+        const float sc = fast_exp2(mv[u] - muse);  // a wave without entries has max = -inf: weight 0
+        l += sc * lv[u];
+#pragma unroll
+        for (int i = 0; i < PER; ++i) o[i] += sc * ov[u][i];
+      }
+      const float inv = l > 0.f ? (p.paged.table ? p.paged.out_scale : 1.f) / l : 0.f;
+      T *op = (T *)p.o.ptr + sq.b * p.o.sb + (int64_t)(h0 + h) * p.o.sh + (int64_t)sq.q_start * p.o.st;
+#pragma unroll
+      for (int i = 0; i < PER; ++i)
+        if (!PAD || lane * PER + i < p.D) op[lane * PER + i] = from_float<T>(o[i] * inv);
+      if (p.lse.ptr && lane == 0)
+        p.lse.ptr[sq.b * p.lse.sb + (h0 + h) * p.lse.sh + (int64_t)sq.q_start * p.lse.st] =
+            l > 0.f ? (mmax + log2f(l)) * kLn2 : -INFINITY;
+    }
+  }
 }
 
 // Merge of the unit partials: one wave per (sequence, q head), lane l owns
@@ -335,7 +415,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
 // make this small kernel latency-bound).
 template <typename T, int D, bool PAD>
 __global__ __launch_bounds__(64) void decode_combine_kernel(const FwdParams p, const float *ws, int unit_blocks,
-                                                            int max_units) {
+                                                            int max_units, int merged_units) {
   constexpr int PER = D / 64;  // dims per lane
   constexpr int MAXU = 8;      // units merged per pass
   const int h = blockIdx.x, b = blockIdx.y, lane = threadIdx.x;
@@ -346,8 +426,10 @@ __global__ __launch_bounds__(64) void decode_combine_kernel(const FwdParams p, c
   if (sq.k_len > 0 && rb < p.csr.num_rows) {
     const int lh = lut_head(p.csr, h, p.Hq, p.Hkv);
     const int n = scalar_load(p.csr.ptr + lh * p.csr.ptr_sh + rb + 1) - scalar_load(p.csr.ptr + lh * p.csr.ptr_sh + rb);
-    units = (n + unit_blocks - 1) / unit_blocks;
+    units = decode_row_units(n, unit_blocks, merged_units > 0 ? merged_units : 1);
   }
+  // rows of at most merged_units units were finished by the partial kernel (merged_units > 0)
+  if (merged_units > 0 && units <= merged_units) return;
   const float *src = ws + ((int64_t)b * p.Hq + h) * max_units * (D + 2);
   float mmax = -INFINITY, l = 0.f, o[PER];
 #pragma unroll
@@ -390,12 +472,7 @@ __global__ __launch_bounds__(64) void decode_combine_kernel(const FwdParams p, c
         l > 0.f ? (mmax + log2f(l)) * kLn2 : -INFINITY;
 }
 
-// Upper bound on the entries of one table row: the caller's hint when given,
-// else the number of column blocks.
-static int decode_max_row_entries(const FwdParams &p) {
-  return p.csr.max_row_entries > 0 ? p.csr.max_row_entries : p.csr.num_rows;
-}
-static int decode_max_units(const FwdParams &p) { return cdiv(decode_max_row_entries(p), decode_unit_blocks()); }
+static int decode_max_units(const FwdParams &p) { return cdiv(decode_max_row_entries(p), decode_unit_blocks(p)); }
 
 bool decode_supported(const FwdParams &p, int dtype) {
   const int ratio = p.Hq / p.Hkv;
@@ -411,19 +488,31 @@ size_t decode_workspace_bytes(const FwdParams &p) {
   return (size_t)p.seqs.batch * p.Hq * decode_max_units(p) * (mfma_tile_width(p.D) + 2) * sizeof(float);
 }
 
-template <typename T, int D, bool PAD, bool SUB, bool PAGED, bool KV8 = false>
-static int launch_decode_td(const FwdParams &p, float *ws, hipStream_t stream) {
-  const int smem = DecSmem<D>::wave_bytes(p.Hq / p.Hkv);
-  const int unit_blocks = decode_unit_blocks(), max_units = decode_max_units(p);
-  DK_REQUIRE(max_units <= 65535, "too many decode units");
-  DK_REQUIRE(!PAGED || unit_blocks <= 16, "paged decode takes at most 16 table entries per unit (DKERNEL_DECODE_UNIT)");
-  hipLaunchKernelGGL((decode_partial_kernel<T, D, PAD, SUB, PAGED, KV8>), dim3(max_units, p.Hkv, p.seqs.batch), dim3(64), smem, stream,
-                     p, ws, unit_blocks, max_units);
+template <typename T, int D, bool PAD, bool SUB, bool PAGED, bool KV8, int W>
+static int launch_decode_tdw(const FwdParams &p, float *ws, hipStream_t stream) {
+  const int smem = W * DecSmem<D>::wave_bytes(p.Hq / p.Hkv);
+  const int unit_blocks = decode_unit_blocks(p), max_units = decode_max_units(p);
+  const int groups = cdiv(max_units, W);
+  DK_REQUIRE(groups <= 65535, "too many decode units");
+  DK_REQUIRE(smem <= 160 * 1024, "decode workgroup needs %d bytes of LDS", smem);
+  DK_ALLOW_DYNAMIC_LDS((decode_partial_kernel<T, D, PAD, SUB, PAGED, KV8, W>), smem);
+  hipLaunchKernelGGL((decode_partial_kernel<T, D, PAD, SUB, PAGED, KV8, W>), dim3(groups, p.Hkv, p.seqs.batch),
+                     dim3(64 * W), smem, stream, p, ws, unit_blocks, max_units);
   DK_HIP_CHECK(hipGetLastError());
+  if (W > 1 && groups == 1) return DK_OK;  // every row was finished inside its workgroup
   hipLaunchKernelGGL((decode_combine_kernel<T, D, PAD>), dim3(p.Hq, p.seqs.batch), dim3(64), 0, stream, p, ws,
-                     unit_blocks, max_units);
+                     unit_blocks, max_units, W > 1 ? W : 0);
   DK_HIP_CHECK(hipGetLastError());
   return DK_OK;
+}
+
+// DKERNEL_DECODE_WAVES=1: one unit per workgroup and every row merged by the second kernel
+// (A/B measurements); default: kDecodeWaves units per workgroup.
+template <typename T, int D, bool PAD, bool SUB, bool PAGED, bool KV8 = false>
+static int launch_decode_td(const FwdParams &p, float *ws, hipStream_t stream) {
+  static const bool single = getenv("DKERNEL_DECODE_WAVES") && atoi(getenv("DKERNEL_DECODE_WAVES")) == 1;
+  if (single) return launch_decode_tdw<T, D, PAD, SUB, PAGED, KV8, 1>(p, ws, stream);
+  return launch_decode_tdw<T, D, PAD, SUB, PAGED, KV8, kDecodeWaves>(p, ws, stream);
 }
 
 template <typename T, bool PAGED>

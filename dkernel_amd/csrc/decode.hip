@@ -1,21 +1,25 @@
-// Split-KV decode kernel for gfx950: one new query token per sequence over
-// padded (left or right) or unpadded 4-D K/V, bf16 / fp16, head_dim 128 or 64,
-// 64 x 64 blocks, grouped-query attention with all q heads of a kv head
-// sharing the look-up-table row.  The step is HBM-bound (every attended K/V
-// byte is read exactly once, for all q heads of the group together), so the
-// design goal is bytes in flight, not FLOPs:
+// Split-KV decode kernels for gfx950: one new query token per sequence over
+// padded (left or right), unpadded, packed or paged K/V, bf16 / fp16 (paged
+// pools also fp8), head_dim a multiple of 8 up to 128, 64 x 64 tiles,
+// grouped-query attention with all q heads of a kv head sharing the
+// look-up-table row.  The step is HBM-bound (every attended K/V byte is read
+// exactly once, for all q heads of the group together), so the design goal is
+// bytes in flight, not FLOPs:
 //
-//   work unit = one wave = at most `unit` consecutive entries of the row of
-//               (sequence, kv head); the number of units of a row follows from
-//               its length on the device, so every wave streams the same
-//               amount of K/V whatever the sequence lengths are (workgroups
-//               beyond a row's unit count exit at once);
+//   work unit = one wave = consecutive entries of the row of (sequence, kv
+//               head); the number of units of a row and the even split of its
+//               entries follow from its length on the device, so waves stream
+//               similar amounts of K/V whatever the sequence lengths are;
+//   workgroup = kDecodeWaves consecutive units of one row (workgroups beyond a
+//               row's unit count exit at once);
 //   wave      = per block: computes S^T = K Q^T (the q heads of the group are the MFMA
 //               columns), softmax, O^T += V^T P^T with LDS transpose reads,
 //               keeping a running (max, sum, O) in registers;
-//   epilogue  = one fp32 partial (O unnormalised, max, sum) per (sequence,
-//               q head, unit) in the caller's workspace; a second small
-//               kernel merges the units, normalises and writes O and LSE.
+//   epilogue  = a row whose units all sit in one workgroup is merged there
+//               through LDS and written as O / LSE; otherwise one fp32
+//               partial (O unnormalised, max, sum) per (sequence, q head,
+//               unit) goes to the caller's workspace and decode_combine_kernel
+//               merges those rows.
 // A wave works on half blocks (32 keys): 2 x 8.5 KB of private LDS tiles and
 // the next half block prefetched into registers, so 8 waves are resident per
 // CU (2 per SIMD, <= 256 VGPRs each): one wave's loads overlap the other's

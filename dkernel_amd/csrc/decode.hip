@@ -161,7 +161,9 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(2, 2))) 
   // PAGED: page numbers of the whole unit in one vector load, four lanes per table entry (a
   // 64-key block spans at most four pages of >= 16 tokens): lane 4 j + s holds the page of keys
   // [s, s + 1) * page_size of entry e0 + j (pages of >= 64 tokens: s = 0 only).  Entries of the
-  // page table beyond the sequence's last token are never read.
+  // page table beyond the sequence's last token are never read; a negative entry inside the
+  // sequence (a caller's mistake: such slots mark unused pages) is read as page 0 rather than
+  // as an address before the pool.
   int my_page = 0;
   if constexpr (PAGED) {
     const int j = lane >> 2, s = lane & 3;
@@ -170,7 +172,7 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(2, 2))) 
       const int col = cols[(e0 + j) * EW];
       const int tok = col * 64 + (ps < 64 ? s * ps : 0);
       if (col >= 0 && tok < sq.k_len && (s == 0 || s * ps < 64))
-        my_page = p.paged.table[b * p.paged.table_sb + (tok >> p.paged.page_shift)];
+        my_page = max(p.paged.table[b * p.paged.table_sb + (tok >> p.paged.page_shift)], 0);
     }
   }
 

@@ -166,7 +166,9 @@ size_t dk_fwd_workspace_bytes(const dk_fwd_args *args);
  * at in-page position t % page_size; a page starts page_stride_k / _v elements
  * after the previous one, tokens and heads inside a page use args->k / v
  * stride_t / stride_h (stride_b is ignored).  page_size is a power of two >= 16.
- * Table entries past a sequence's last token are never read.  args->seqs
+ * Table entries past a sequence's last token are never read; entries before it
+ * must name pages of the pools (the library cannot check their upper bound; a
+ * negative one is read as page 0).  args->seqs
  * gives the lengths as for padded decode (q one token per sequence, k_starts 0,
  * k_ends the context lengths, max_k_len the table's capacity in tokens) and
  * args->workspace must hold dk_fwd_workspace_bytes(args).  No counterpart in

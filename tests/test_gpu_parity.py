@@ -316,6 +316,22 @@ def test_paged_decode(page_size, bs, D, head_major):
         assert_close(f"LSE[{i}]", lse[i], rl, atol=LSE_TOL, rtol=0)
 
 
+def test_paged_decode_negative_table_entry_reads_page_zero():
+    """A page-table slot marked unused (-1) inside a sequence is a caller's mistake; the kernel
+    reads page 0 for it instead of an address before the pools."""
+    B, Hq, Hkv, D, Lmax, page = 2, 8, 2, 128, 256, 16
+    g = torch.Generator().manual_seed(20)
+    q = torch.randn(B, Hq, D, generator=g).to(torch.bfloat16).to(DEV)
+    k_pool = torch.randn(4, page, Hkv, D, generator=g).to(torch.bfloat16).to(DEV)
+    v_pool = torch.randn(4, page, Hkv, D, generator=g).to(torch.bfloat16).to(DEV)
+    table = torch.full((B, Lmax // page), -1, dtype=torch.int32, device=DEV)
+    mod = _module(Hq, Lmax, 64, 2, 4, num_kv_heads=Hkv)
+    out = mod.paged_decode(q, k_pool, v_pool, table, torch.ones(B, dtype=torch.int32, device=DEV), 0.1)
+    # one key per sequence: O = V of token 0 of page 0
+    want = v_pool[0, 0].repeat_interleave(Hq // Hkv, dim=0)[None].expand(B, Hq, D)
+    assert torch.equal(out, want)
+
+
 @pytest.mark.parametrize("page_size,bs,D,dtype", [(16, 64, 128, torch.bfloat16), (64, 128, 64, torch.float16)])
 def test_paged_decode_fp8_cache(page_size, bs, D, dtype):
     """Paged decode over OCP e4m3 K/V pools with per-tensor scales: the oracle attends to the

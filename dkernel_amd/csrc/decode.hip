@@ -11,7 +11,9 @@
 //               entries follow from its length on the device, so waves stream
 //               similar amounts of K/V whatever the sequence lengths are;
 //   workgroup = kDecodeWaves consecutive units of one row (workgroups beyond a
-//               row's unit count exit at once);
+//               row's unit count exit at once; a row that needs several
+//               workgroups is cut into a whole number of them, so that none
+//               holds LDS and wave slots for idle waves);
 //   wave      = per block: computes S^T = K Q^T (the q heads of the group are the MFMA
 //               columns), softmax, O^T += V^T P^T with LDS transpose reads,
 //               keeping a running (max, sum, O) in registers;
@@ -59,11 +61,14 @@ static int decode_unit_blocks(const FwdParams &p) {
 
 // Units a row of n table entries is cut into: as many as the unit size asks for, and at least
 // the waves of one workgroup (one entry each at worst), so that every wave of the workgroup that
-// finishes a row streams a share of it.  Used by both kernels.
+// finishes a row streams a share of it.  A row that needs more than one workgroup gets a whole
+// number of them: a workgroup with a single busy wave would hold the LDS and the wave slots of
+// four.  Used by both kernels.
 __host__ __device__ inline int decode_row_units(int n, int unit_blocks, int waves) {
   const int by_size = (n + unit_blocks - 1) / unit_blocks;
   const int by_waves = n < waves ? n : waves;
-  return by_size > by_waves ? by_size : by_waves;
+  const int units = by_size > by_waves ? by_size : by_waves;
+  return units > waves ? (units + waves - 1) / waves * waves : units;
 }
 
 template <int D>
@@ -231,7 +236,7 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(2, 2))) 
   };
   // the first K/V request goes out before anything else touches memory
   int col_cur = 0, bits_cur = 0;
-  if (active) {
+  if (e0 < e1) {  // (an even split can leave the last units of a row without entries: neutral partials)
     if constexpr (SUB)
       scalar_load2(cols + e0 * EW, cols + e0 * EW + 1, col_cur, bits_cur);
     else
@@ -478,7 +483,11 @@ __global__ __launch_bounds__(64) void decode_combine_kernel(const FwdParams p, c
         l > 0.f ? (mmax + log2f(l)) * kLn2 : -INFINITY;
 }
 
-static int decode_max_units(const FwdParams &p) { return cdiv(decode_max_row_entries(p), decode_unit_blocks(p)); }
+// Unit slots per (sequence, q head) in the workspace: the longest row's units (rows that fit one
+// workgroup keep their partials in LDS).
+static int decode_max_units(const FwdParams &p) {
+  return decode_row_units(decode_max_row_entries(p), decode_unit_blocks(p), kDecodeWaves);
+}
 
 bool decode_supported(const FwdParams &p, int dtype) {
   const int ratio = p.Hq / p.Hkv;

@@ -114,7 +114,6 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(2, 2))) 
   using S = DecSmem<D>;
   constexpr int KS = D / 16, DT = D / 32, CPR = D / 8;
   // SUB: table entries are (column, bit mask over the pattern blocks inside the 64 x 64 tile)
-  static_assert(!SUB || !PAD, "sub-block masks: plain tiles only");
   constexpr int EW = SUB ? 2 : 1;  // ints per table entry
   extern __shared__ __align__(16) char smem_all[];
 
@@ -495,7 +494,7 @@ bool decode_supported(const FwdParams &p, int dtype) {
                           (p.csr.num_heads == p.Hq && p.csr.group % ratio == 0);
   return (dtype == DK_BF16 || dtype == DK_F16) && mfma_head_dim_ok(p.D) && p.csr.block_rows == 64 &&
          p.csr.block_cols == 64 && p.vec_ok &&
-         (p.csr.entry_width == 1 || (p.csr.sub_block != 0 && (p.D == 64 || p.D == 128))) &&
+         (p.csr.entry_width == 1 || p.csr.sub_block != 0) &&
          (p.seqs.packed ? (p.seqs.packed & 2) != 0 : p.seqs.max_q_len == 1) && ratio <= 32 && shared_row && p.causal;
 }
 
@@ -532,9 +531,12 @@ static int launch_decode_td(const FwdParams &p, float *ws, hipStream_t stream) {
 
 template <typename T, bool PAGED>
 static int launch_decode_tp(const FwdParams &p, float *ws, hipStream_t stream) {
-  if (p.csr.sub_block)  // entries carry a bit mask over the pattern's 16- or 32-token blocks
-    return p.D == 128 ? launch_decode_td<T, 128, false, true, PAGED>(p, ws, stream)
-                      : launch_decode_td<T, 64, false, true, PAGED>(p, ws, stream);
+  if (p.csr.sub_block) {  // entries carry a bit mask over the pattern's 16- or 32-token blocks
+    if (p.D == 128) return launch_decode_td<T, 128, false, true, PAGED>(p, ws, stream);
+    if (p.D == 64) return launch_decode_td<T, 64, false, true, PAGED>(p, ws, stream);
+    return p.D > 64 ? launch_decode_td<T, 128, true, true, PAGED>(p, ws, stream)
+                    : launch_decode_td<T, 64, true, true, PAGED>(p, ws, stream);
+  }
   if (p.D == 128) return launch_decode_td<T, 128, false, false, PAGED>(p, ws, stream);
   if (p.D == 64) return launch_decode_td<T, 64, false, false, PAGED>(p, ws, stream);
   return p.D > 64 ? launch_decode_td<T, 128, true, false, PAGED>(p, ws, stream)

@@ -53,7 +53,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, D == 64 
   constexpr int KS = D / 16, DT = D / 32;
   constexpr int STAGE = 2 * TL::kBytes;
   // SUB: table entries are (column, bit mask over the pattern blocks inside the 64 x 64 tile)
-  static_assert(!SUB || !PAD, "sub-block masks: plain tiles only");
   constexpr int EW = SUB ? 2 : 1;  // ints per table entry
   extern __shared__ __align__(16) char smem[];
 
@@ -327,7 +326,6 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   constexpr int KS = D / 16, DT = D / 32;
   constexpr int LPT = 2 * TileLoader<D, NT>::kChunks + 1;  // load instructions per wave per block
   // SUB: table entries are (row block, bit mask over the pattern blocks inside the 64 x 64 tile)
-  static_assert(!SUB || !PAD, "sub-block masks: plain tiles only");
   constexpr int EW = SUB ? 2 : 1;  // ints per table entry
   extern __shared__ __align__(16) char smem[];
 
@@ -640,27 +638,35 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 template __global__ void mfma_dq_kernel<bf16_t, 128, false, false>(const BwdParams, int);
 template __global__ void mfma_dq_kernel<bf16_t, 128, true, false>(const BwdParams, int);
 template __global__ void mfma_dq_kernel<bf16_t, 128, false, true>(const BwdParams, int);
+template __global__ void mfma_dq_kernel<bf16_t, 128, true, true>(const BwdParams, int);
 template __global__ void mfma_dq_kernel<bf16_t, 64, false, false>(const BwdParams, int);
 template __global__ void mfma_dq_kernel<bf16_t, 64, true, false>(const BwdParams, int);
 template __global__ void mfma_dq_kernel<bf16_t, 64, false, true>(const BwdParams, int);
+template __global__ void mfma_dq_kernel<bf16_t, 64, true, true>(const BwdParams, int);
 template __global__ void mfma_dq_kernel<f16_t, 128, false, false>(const BwdParams, int);
 template __global__ void mfma_dq_kernel<f16_t, 128, true, false>(const BwdParams, int);
 template __global__ void mfma_dq_kernel<f16_t, 128, false, true>(const BwdParams, int);
+template __global__ void mfma_dq_kernel<f16_t, 128, true, true>(const BwdParams, int);
 template __global__ void mfma_dq_kernel<f16_t, 64, false, false>(const BwdParams, int);
 template __global__ void mfma_dq_kernel<f16_t, 64, true, false>(const BwdParams, int);
 template __global__ void mfma_dq_kernel<f16_t, 64, false, true>(const BwdParams, int);
+template __global__ void mfma_dq_kernel<f16_t, 64, true, true>(const BwdParams, int);
 template __global__ void mfma_dkdv_kernel<bf16_t, 128, false, false>(const BwdParams, int);
 template __global__ void mfma_dkdv_kernel<bf16_t, 128, true, false>(const BwdParams, int);
 template __global__ void mfma_dkdv_kernel<bf16_t, 128, false, true>(const BwdParams, int);
+template __global__ void mfma_dkdv_kernel<bf16_t, 128, true, true>(const BwdParams, int);
 template __global__ void mfma_dkdv_kernel<bf16_t, 64, false, false>(const BwdParams, int);
 template __global__ void mfma_dkdv_kernel<bf16_t, 64, true, false>(const BwdParams, int);
 template __global__ void mfma_dkdv_kernel<bf16_t, 64, false, true>(const BwdParams, int);
+template __global__ void mfma_dkdv_kernel<bf16_t, 64, true, true>(const BwdParams, int);
 template __global__ void mfma_dkdv_kernel<f16_t, 128, false, false>(const BwdParams, int);
 template __global__ void mfma_dkdv_kernel<f16_t, 128, true, false>(const BwdParams, int);
 template __global__ void mfma_dkdv_kernel<f16_t, 128, false, true>(const BwdParams, int);
+template __global__ void mfma_dkdv_kernel<f16_t, 128, true, true>(const BwdParams, int);
 template __global__ void mfma_dkdv_kernel<f16_t, 64, false, false>(const BwdParams, int);
 template __global__ void mfma_dkdv_kernel<f16_t, 64, true, false>(const BwdParams, int);
 template __global__ void mfma_dkdv_kernel<f16_t, 64, false, true>(const BwdParams, int);
+template __global__ void mfma_dkdv_kernel<f16_t, 64, true, true>(const BwdParams, int);
 
 // Sum of the per-q-head dK / dV partials over each kv group (head_split mode).  One thread
 // per 8 head dims of one (batch, kv head, key): blockIdx.y = 0 sums dK, 1 sums dV.
@@ -708,7 +714,7 @@ size_t mfma_bwd_workspace_bytes(const BwdParams &p) {
 bool mfma_bwd_supported(const BwdParams &p, int dtype) {
   return (dtype == DK_BF16 || dtype == DK_F16) && mfma_head_dim_ok(p.D) && p.csr.block_rows == 64 &&
          p.csr.block_cols == 64 && p.csr.sub_block == p.csc.sub_block &&
-         (p.csr.sub_block ? (p.D == 64 || p.D == 128) : (p.csr.entry_width == 1 && p.csc.entry_width == 1)) &&
+         (p.csr.sub_block != 0 || (p.csr.entry_width == 1 && p.csc.entry_width == 1)) &&
          p.csc.block_rows == 64 && p.csc.block_cols == 64 &&
          p.vec_ok;
 }
@@ -754,9 +760,12 @@ static int launch_bwd_td(const BwdParams &p, void *workspace, size_t workspace_b
 // head dims below the tile width (64 or 128) run the zero-padded instantiation
 template <typename T>
 static int launch_bwd_t(const BwdParams &p, void *ws, size_t ws_bytes, hipStream_t stream) {
-  if (p.csr.sub_block)  // entries carry a bit mask over the pattern's 16- or 32-token blocks
-    return p.D == 128 ? launch_bwd_td<T, 128, false, true>(p, ws, ws_bytes, stream)
-                      : launch_bwd_td<T, 64, false, true>(p, ws, ws_bytes, stream);
+  if (p.csr.sub_block) {  // entries carry a bit mask over the pattern's 16- or 32-token blocks
+    if (p.D == 128) return launch_bwd_td<T, 128, false, true>(p, ws, ws_bytes, stream);
+    if (p.D == 64) return launch_bwd_td<T, 64, false, true>(p, ws, ws_bytes, stream);
+    return p.D > 64 ? launch_bwd_td<T, 128, true, true>(p, ws, ws_bytes, stream)
+                    : launch_bwd_td<T, 64, true, true>(p, ws, ws_bytes, stream);
+  }
   if (p.D == 128) return launch_bwd_td<T, 128, false, false>(p, ws, ws_bytes, stream);
   if (p.D == 64) return launch_bwd_td<T, 64, false, false>(p, ws, ws_bytes, stream);
   return p.D > 64 ? launch_bwd_td<T, 128, true, false>(p, ws, ws_bytes, stream)

@@ -52,7 +52,7 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
 
   static_assert(!RP || G == 2, "row pairs: two wave pairs, one q tile each");
   // SUB: table entries are (column, bit mask over the pattern blocks inside the 64 x 64 tile)
-  static_assert(!SUB || (!RP && !PAD), "sub-block masks: plain tiles only");
+  static_assert(!SUB || !RP, "sub-block masks: one q tile per workgroup");
   constexpr int EW = SUB ? 2 : 1;  // ints per table entry
   SeqInfo sq;
   int tile;
@@ -645,14 +645,18 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
   template __global__ void mfma_fwd_kernel<T, D, 2, PAD, true>(const FwdParams, int);  \
   template __global__ void mfma_fwd_kernel<T, D, 4, PAD, false>(const FwdParams, int); \
   template __global__ void mfma_fwd_pipe_kernel<T, D, 1, PAD>(const FwdParams, int);
-#define DK_INSTANTIATE_FWD_SUB(T, D)                                                                  \
-  template __global__ void mfma_fwd_kernel<T, D, 1, false, false, true>(const FwdParams, int); \
-  template __global__ void mfma_fwd_kernel<T, D, 2, false, false, true>(const FwdParams, int); \
-  template __global__ void mfma_fwd_kernel<T, D, 4, false, false, true>(const FwdParams, int);
-DK_INSTANTIATE_FWD_SUB(bf16_t, 128)
-DK_INSTANTIATE_FWD_SUB(bf16_t, 64)
-DK_INSTANTIATE_FWD_SUB(f16_t, 128)
-DK_INSTANTIATE_FWD_SUB(f16_t, 64)
+#define DK_INSTANTIATE_FWD_SUB(T, D, PAD)                                                    \
+  template __global__ void mfma_fwd_kernel<T, D, 1, PAD, false, true>(const FwdParams, int); \
+  template __global__ void mfma_fwd_kernel<T, D, 2, PAD, false, true>(const FwdParams, int); \
+  template __global__ void mfma_fwd_kernel<T, D, 4, PAD, false, true>(const FwdParams, int);
+DK_INSTANTIATE_FWD_SUB(bf16_t, 128, false)
+DK_INSTANTIATE_FWD_SUB(bf16_t, 64, false)
+DK_INSTANTIATE_FWD_SUB(f16_t, 128, false)
+DK_INSTANTIATE_FWD_SUB(f16_t, 64, false)
+DK_INSTANTIATE_FWD_SUB(bf16_t, 128, true)
+DK_INSTANTIATE_FWD_SUB(bf16_t, 64, true)
+DK_INSTANTIATE_FWD_SUB(f16_t, 128, true)
+DK_INSTANTIATE_FWD_SUB(f16_t, 64, true)
 #undef DK_INSTANTIATE_FWD_SUB
 DK_INSTANTIATE_FWD(bf16_t, 128, false)
 DK_INSTANTIATE_FWD(bf16_t, 64, false)
@@ -679,7 +683,7 @@ static int fwd_group(const FwdParams &p) {
 bool mfma_fwd_supported(const FwdParams &p, int dtype) {
   return (dtype == DK_BF16 || dtype == DK_F16) && mfma_head_dim_ok(p.D) && p.csr.block_rows == 64 &&
          p.csr.block_cols == 64 && p.vec_ok &&
-         (p.csr.entry_width == 1 || (p.csr.sub_block != 0 && (p.D == 64 || p.D == 128)));
+         (p.csr.entry_width == 1 || p.csr.sub_block != 0);
 }
 
 template <typename T, int D, int G, bool PAD>
@@ -743,32 +747,34 @@ static int launch_tdp(const FwdParams &p, dim3 grid, int tiles_y, hipStream_t st
 }
 
 // Tables whose entries carry a bit mask over the pattern's 16- or 32-token blocks inside each
-// 64 x 64 tile: the plain kernel with the mask applied to S (no row pairs, no padded head dims).
-template <typename T, int D, int G>
+// 64 x 64 tile: the plain kernel with the mask applied to S (no row pairs).
+template <typename T, int D, int G, bool PAD>
 static int launch_sub_g(const FwdParams &p, dim3 grid, int tiles_y, hipStream_t stream) {
   constexpr int smem = 2 * FwdSmem<D>::kStage;
-  DK_ALLOW_DYNAMIC_LDS((mfma_fwd_kernel<T, D, G, false, false, true>), smem);
+  DK_ALLOW_DYNAMIC_LDS((mfma_fwd_kernel<T, D, G, PAD, false, true>), smem);
   grid.x = p.Hq / G;
-  hipLaunchKernelGGL((mfma_fwd_kernel<T, D, G, false, false, true>), grid, dim3(128 * G), smem, stream, p, tiles_y);
+  hipLaunchKernelGGL((mfma_fwd_kernel<T, D, G, PAD, false, true>), grid, dim3(128 * G), smem, stream, p, tiles_y);
   DK_HIP_CHECK(hipGetLastError());
   return DK_OK;
 }
 
-template <typename T, int D>
+template <typename T, int D, bool PAD>
 static int launch_sub(const FwdParams &p, dim3 grid, int tiles_y, hipStream_t stream) {
   const int group = D == 64 && fwd_group(p) == 4 ? 2 : fwd_group(p);  // as in launch_tdp
   switch (group) {
-    case 4: return launch_sub_g<T, D, 4>(p, grid, tiles_y, stream);
-    case 2: return launch_sub_g<T, D, 2>(p, grid, tiles_y, stream);
-    default: return launch_sub_g<T, D, 1>(p, grid, tiles_y, stream);
+    case 4: return launch_sub_g<T, D, 4, PAD>(p, grid, tiles_y, stream);
+    case 2: return launch_sub_g<T, D, 2, PAD>(p, grid, tiles_y, stream);
+    default: return launch_sub_g<T, D, 1, PAD>(p, grid, tiles_y, stream);
   }
 }
 
 // head dims below the tile width (64 or 128) run the zero-padded instantiation
 template <typename T>
 static int launch_t(const FwdParams &p, dim3 grid, int tiles_y, hipStream_t stream) {
-  if (p.csr.sub_block) {
-    return p.D == 128 ? launch_sub<T, 128>(p, grid, tiles_y, stream) : launch_sub<T, 64>(p, grid, tiles_y, stream);
+  if (p.csr.sub_block) {  // entries carry a bit mask over the pattern's 16- or 32-token blocks
+    if (p.D == 128) return launch_sub<T, 128, false>(p, grid, tiles_y, stream);
+    if (p.D == 64) return launch_sub<T, 64, false>(p, grid, tiles_y, stream);
+    return p.D > 64 ? launch_sub<T, 128, true>(p, grid, tiles_y, stream) : launch_sub<T, 64, true>(p, grid, tiles_y, stream);
   }
   if (p.D == 128) return launch_tdp<T, 128, false>(p, grid, tiles_y, stream);
   if (p.D == 64) return launch_tdp<T, 64, false>(p, grid, tiles_y, stream);

@@ -254,8 +254,8 @@ class SparseAttention(torch.nn.Module):
         kv heads, dim), page_size a power of two >= 16; block_table: int32 (batch, pages per
         sequence); context_lens: int32 (batch,) keys per sequence including the new token's.
         Pools of dtype torch.float8_e4m3fn hold K / k_scale and V / v_scale (head_dim 64 / 128,
-        blocks of at least 64).  Needs the matrix-core decode kernels (bf16 / fp16, head_dim a multiple of 8 up to 128;
-        with blocks of 16 / 32: head_dim 64 or 128).  No counterpart in the reference."""
+        blocks of at least 64).  Needs the matrix-core decode kernels (bf16 / fp16, head_dim a multiple
+        of 8 up to 128).  No counterpart in the reference."""
         from .ops import paged_decode_attn
         assert self.kwargs.get('causal', True), "paged decode is causal"
         if self.kernel_tile is not None:

@@ -125,6 +125,11 @@ def test_matrix_core_kernels_take_padded_dims_and_split_blocks():
         run_fwd_bwd(2, 8, 2, 1000, 128, torch.bfloat16, 16, 5, 7)
         run_fwd_bwd(1, 4, 4, 777, 64, torch.float16, 32, 3, 3)
         run_fwd_bwd(1, 2, 2, 512, 128, torch.bfloat16, 16, 3, 9, causal=False)
+        # ... together with head dims below the tile width
+        run_fwd_bwd(2, 8, 2, 1000, 96, torch.bfloat16, 16, 5, 7)
+        run_fwd_bwd(1, 4, 4, 777, 40, torch.float16, 32, 3, 3)
+        run_fwd_bwd(1, 4, 1, 640, 120, torch.bfloat16, 32, 2, 5)
+        run_fwd_bwd(1, 2, 2, 512, 80, torch.float16, 16, 3, 9, causal=False)
         with pytest.raises(Exception, match="no MFMA"):
             run_fwd_bwd(1, 2, 2, 256, 160, torch.bfloat16, 64, 2, 4)
     finally:
@@ -273,9 +278,20 @@ def test_decode_head_dims_below_tile_width(impl, D, left):
     _decode_case(64, None, left, D)
 
 
+@pytest.mark.parametrize("bs,D,left", [(16, 96, True), (32, 40, False)])
+def test_decode_small_blocks_with_padded_head_dims(bs, D, left):
+    """Blocks of 16 / 32 (masked tiles) and a head dim below the tile width, matrix-core kernels forced."""
+    ops.set_impl("mfma")
+    try:
+        _decode_case(bs, None, left, D)
+    finally:
+        ops.set_impl("auto")
+
+
 @pytest.mark.parametrize("page_size,bs,D,head_major", [(16, 64, 128, False), (32, 64, 128, True), (64, 64, 96, False),
                                                         (128, 64, 128, False), (16, 16, 128, False),
-                                                        (32, 128, 64, True), (256, 32, 128, False)])
+                                                        (32, 128, 64, True), (256, 32, 128, False),
+                                                        (16, 16, 96, False), (64, 32, 40, True)])
 def test_paged_decode(page_size, bs, D, head_major):
     """Single-token decode over a paged K/V cache: pages scattered in the pools, table rows padded
     with -1 past each sequence, pools token-major or head-major inside a page; against the oracle

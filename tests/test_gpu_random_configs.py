@@ -148,8 +148,6 @@ def test_random_inference_config_matches_generic_kernels_and_oracle(seed):
     dtype = torch.bfloat16 if rng.random() < 0.7 else torch.float16
     mode = str(rng.choice(["left", "right", "packed", "packed_decode", "left_decode", "right_decode", "chunked",
                            "paged_decode"]))
-    if mode == "paged_decode" and bs < 64 and D not in (64, 128):
-        D = 64  # masked tiles (blocks of 16 / 32) exist for head_dim 64 / 128 only, and paged K/V has no generic path
     nseq = int(rng.integers(1, 6))
     Lmax = int(rng.choice([256, 512, 1024]))
     lens = [int(rng.integers(1, Lmax + 1)) for _ in range(nseq)]

@@ -50,10 +50,8 @@ static int decode_max_row_entries(const FwdParams &p) {
 // units (about 1024 waves in total).  At most 16 (the paged path keeps a unit's page numbers in
 // the lanes of one register).  DKERNEL_DECODE_UNIT overrides.
 static int decode_unit_blocks(const FwdParams &p) {
-  if (const char *env = getenv("DKERNEL_DECODE_UNIT")) {
-    const int v = atoi(env);
-    if (v >= 1 && v <= 16) return v;
-  }
+  static const int forced = getenv("DKERNEL_DECODE_UNIT") ? atoi(getenv("DKERNEL_DECODE_UNIT")) : 0;  // read once
+  if (forced >= 1 && forced <= 16) return forced;
   const int rows = p.seqs.batch * p.Hkv;
   const int units_per_row = std::max(kDecodeWaves, cdiv(1024, rows > 0 ? rows : 1));
   return std::min(16, std::max(2, cdiv(decode_max_row_entries(p), units_per_row)));

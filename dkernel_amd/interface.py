@@ -17,6 +17,7 @@ from torch import Tensor
 from .ops import _sparse_attention
 from .utils import (dense_to_ccol_row, dense_to_crow_col, get_sparse_attn_mask, is_kv_cache_efficient,
                     masked_tile_tables, merge_split_fwd_kernel_blocks, multiple_of, split_tile_tables,
+                    tile_sizes_keep_pattern,
                     verify_sparse_pattern, zero_stride)
 
 _KERNEL_TILE = 64  # q and k tile of the matrix-core kernels
@@ -48,12 +49,13 @@ class SparseAttention(torch.nn.Module):
     block_m, block_n: kernel tile sizes on q and k (powers of 2, >= 16).
         Default block_m = max(block_size, 64) if causal else block_size,
         block_n = block_size; the attributes and the `layout_*` buffers follow
-        these defaults as in the reference.  When both are left unset and
-        block_size is not 64, the kernels themselves read extra tables built for
-        their 64 x 64 tiles (`kernel_*`: larger blocks split; `masked_*`:
-        smaller blocks as tiles with a bit mask; `exact_csr_*`: unmerged tiles
-        for the generic kernels), which follow the pattern exactly.  Explicit
-        values are honoured as given (generic kernels).
+        these values as in the reference.  The kernels themselves read extra
+        tables built for their 64 x 64 tiles (`kernel_*`: larger blocks split;
+        `masked_*`: smaller blocks as tiles with a bit mask; `exact_csr_*`:
+        unmerged tiles), which follow the pattern exactly -- unless block_m is
+        given and merging q rows widens the pattern (a later pattern row of a
+        merged tile holds a column an earlier one lacks): then the merged table
+        is used as given, on the generic kernels.
     kwargs: "out" (output tensor), "d_splits" (accepted, unused), "inference"
         (skip saving the log-sum-exp for backward; default: no input needs grad).
 
@@ -83,12 +85,7 @@ class SparseAttention(torch.nn.Module):
         _check_block_size(block_m, "block_m")
         _check_block_size(block_n, "block_n")
 
-        # Patterns with blocks larger than the 64 x 64 tile of the matrix-core kernels run on
-        # tables split to that tile, unless the caller fixes the tile sizes.
-        split_for_kernels = block_m is None and block_n is None and block_size > _KERNEL_TILE
-        # ... and patterns with smaller blocks on tile tables whose entries carry a bit mask over
-        # the pattern blocks inside the tile
-        mask_for_kernels = block_m is None and block_n is None and block_size < _KERNEL_TILE
+        explicit_tiles = block_m is not None or block_n is not None
         if block_m is None:
             block_m = max(block_size, 64) if causal else block_size
         if block_n is None:
@@ -119,6 +116,19 @@ class SparseAttention(torch.nn.Module):
             # merged q tiles are a causal-only optimisation
             assert self.block_m <= block_size
             assert self.block_n <= block_size
+
+        # Tile sizes given by the caller are honoured in the layout_* buffers.  The kernels run
+        # 64 x 64 tiles of their own (below) whenever that attends the same blocks, i.e. always
+        # except for a merged-row table over a pattern in which a later row of a merged tile
+        # holds a column that an earlier one lacks.
+        own_tiles = not explicit_tiles or tile_sizes_keep_pattern(block_size, sparse_pattern, self.block_m,
+                                                                  self.block_n, causal)
+        # patterns with blocks larger than the 64 x 64 tile of the matrix-core kernels run on
+        # tables split to that tile
+        split_for_kernels = own_tiles and block_size > _KERNEL_TILE
+        # ... and patterns with smaller blocks on tile tables whose entries carry a bit mask over
+        # the pattern blocks inside the tile
+        mask_for_kernels = own_tiles and block_size < _KERNEL_TILE
 
         layout_csr = list(merge_split_fwd_kernel_blocks(block_size, sparse_pattern,
                                                         self.block_m, self.block_n, causal=causal))
@@ -166,13 +176,16 @@ class SparseAttention(torch.nn.Module):
         # layout_csr_* buffers keep that table; the kernels follow the pattern itself: unmerged
         # tiles for the generic kernels, masked 64 x 64 tiles for the matrix-core kernels.
         self.exact_tile = None
-        if mask_for_kernels and self.block_m != block_size:
+        if own_tiles and not split_for_kernels and (self.block_m != block_size or self.block_n != block_size):
             exact = list(dense_to_crow_col(sparse_pattern))
             if exact[0].dim() == 1:
                 exact = [x[None] for x in exact]
             if exact[0].size(0) == 1:
                 exact = [zero_stride(x) for x in exact]
             self.exact_tile = block_size
+            crow = exact[0]
+            self.lut_max_row = int((crow[:, 1:] - crow[:, :-1]).max()) if crow.size(1) > 1 else 0
+            self.kwargs['lut_max_row'] = self.lut_max_row
             self.register_buffer("exact_csr_crow", exact[0].to(torch.int32), persistent=False)
             self.register_buffer("exact_csr_col", exact[1].to(torch.int32), persistent=False)
 
@@ -264,6 +277,9 @@ class SparseAttention(torch.nn.Module):
         elif self.mask_tile is not None:
             layout = (self.masked_csr_crow, self.masked_csr_col, self.mask_tile, self.mask_tile, self.block_size)
             max_row = self.mask_lut_max_row
+        elif self.exact_tile is not None:
+            layout = (self.exact_csr_crow, self.exact_csr_col, self.exact_tile, self.exact_tile)
+            max_row = self.lut_max_row
         else:
             layout = (self.layout_csr_crow, self.layout_csr_col, self.block_m, self.block_n)
             max_row = self.lut_max_row

@@ -250,6 +250,30 @@ def merge_split_fwd_kernel_blocks(block_size: int, sparse_pattern: Tensor, block
     return dense_to_crow_col(out.to(sparse_pattern.device), include_values=merged)
 
 
+def tile_sizes_keep_pattern(block_size: int, sparse_pattern: Tensor, block_m: int, block_n: int,
+                            causal: bool = True) -> bool:
+    """Whether a table of block_m x block_n kernel tiles attends exactly the pattern's own
+    blocks.  Splitting never changes what is attended; merging q rows does when a column is
+    held only by a later pattern row of a merged tile, because every row of the tile up to
+    the last holder then attends it (dkernel/utils.py:299-308).  Blocks entirely above the
+    token diagonal do not count (the kernels mask them)."""
+    out, merged = _tile_pattern(block_size, sparse_pattern, block_m, block_n, causal)
+    if not merged:
+        return True
+    p = (sparse_pattern != 0).to("cpu")
+    H, M, N = p.shape
+    mm, split_n = block_m // block_size, block_size // block_n
+    om, on = out.shape[1:]
+    # rows s of merged tile i attend column j iff s * block_size < out[i, j]
+    sub = torch.arange(mm)[None, None, :, None] * block_size
+    eff = (out[:, :, None, :] > sub).reshape(H, om * mm, on)[:, :M]
+    own = p.repeat_interleave(split_n, dim=2)[:, :, :on]
+    rows = torch.arange(M)[:, None]
+    cols = torch.arange(on)[None, :]
+    visible = cols * block_n < (rows + 1) * block_size if causal else torch.ones(M, on, dtype=torch.bool)
+    return bool(((eff == own) | ~visible[None]).all())
+
+
 def split_tile_tables(block_size: int, sparse_pattern: Tensor, tile: int,
                       causal: bool = True) -> Tuple[Tuple[Tensor, Tensor], Tuple[Tensor, Tensor]]:
     """CSR and CSC tables of a pattern whose blocks are split into tile x tile

@@ -181,6 +181,18 @@ def test_kernel_tile_sizes(impl, bs, bm, bn):
     run_fwd_bwd(1, 2, 2, 1024, 128, torch.bfloat16, bs, 1, 4, block_m=bm, block_n=bn)
 
 
+@pytest.mark.parametrize("bs,bm,bn", [(16, 128, 16), (64, 128, 32), (32, 64, 32), (128, 128, 64)])
+def test_kernel_tile_sizes_on_the_matrix_cores(bs, bm, bn):
+    """Tile sizes given by the caller do not keep a local-stride pattern off the matrix-core
+    kernels (forced here): they run their own 64 x 64 tiles over the same blocks."""
+    ops.set_impl("mfma")
+    try:
+        run_fwd_bwd(1, 4, 2, 1024, 128, torch.bfloat16, bs, 2, 4, block_m=bm, block_n=bn)
+        run_fwd_bwd(1, 2, 2, 1000, 96, torch.float16, bs, 1, 3, block_m=bm, block_n=bn)
+    finally:
+        ops.set_impl("auto")
+
+
 @pytest.mark.parametrize("bs,D,dtype", [(128, 128, torch.bfloat16), (256, 128, torch.bfloat16),
                                         (128, 64, torch.float16)])
 def test_large_blocks_run_on_split_tiles(impl, bs, D, dtype):

@@ -182,8 +182,10 @@ def test_large_blocks_get_split_kernel_tables(bs, causal):
     got_csc = U.ccol_row_to_dense(m.kernel_csc_ccol, m.kernel_csc_row, torch.uint8).numpy() != 0
     assert np.array_equal(got_csr, want) and np.array_equal(got_csc, want)
     assert m.lut_max_row == int(want.sum(-1).max())
-    # explicit tile sizes are honoured as given
-    assert LocalStrideSparseAttention(H, L, bs, 2, 4, causal=causal, block_m=bs, block_n=64).kernel_tile is None
+    # explicit tile sizes shape the layout_* buffers; the kernels still get their own tiles
+    e = LocalStrideSparseAttention(H, L, bs, 2, 4, causal=causal, block_m=bs, block_n=64)
+    assert e.kernel_tile == 64 and (e.block_m, e.block_n) == (bs, 64)
+    assert e.layout_csr_crow.shape[-1] == L // bs + 1 and torch.equal(e.kernel_csr_col, m.kernel_csr_col)
     assert LocalStrideSparseAttention(H, L, 64, 2, 4, causal=causal).kernel_tile is None
 
 
@@ -217,8 +219,48 @@ def test_small_blocks_get_masked_tile_tables(bs, causal):
     assert np.array_equal(rebuild(m.masked_csc_ccol, m.masked_csc_row, True), want)
     crow = m.masked_csr_crow.numpy()
     assert m.mask_lut_max_row == int((crow[:, 1:] - crow[:, :-1]).max())
-    # explicit tile sizes are honoured as given
-    assert LocalStrideSparseAttention(H, L, bs, 3, 5, causal=causal, block_m=bs, block_n=bs).mask_tile is None
+    # explicit tile sizes shape the layout_* buffers; the kernels still get their own tiles
+    e = LocalStrideSparseAttention(H, L, bs, 3, 5, causal=causal, block_m=bs, block_n=bs)
+    assert e.mask_tile == 64 and e.exact_tile is None and e.layout_csr_crow.shape[-1] == e.max_seqlen // bs + 1
+
+
+def test_tile_sizes_given_by_the_caller_keep_the_pattern_or_not():
+    """Explicit block_m / block_n only re-tile a local-stride pattern (the kernels may then run
+    their own 64 x 64 tiles); a merged-row table over a pattern whose later row holds a column the
+    earlier row lacks attends more than the pattern (checked against a brute-force expansion)."""
+    for bs, bm, bn in [(16, 128, 16), (64, 128, 32), (16, 64, 16), (32, 32, 16), (64, 64, 64)]:
+        pat = torch.from_numpy(np.asarray(OL.block_mask(4, 1024, bs, 2, 3))).to(torch.uint8)
+        assert U.tile_sizes_keep_pattern(bs, pat, bm, bn, True)
+        mod = LocalStrideSparseAttention(4, 1024, bs, 2, 3, block_m=bm, block_n=bn)
+        assert (mod.block_m, mod.block_n) == (bm, bn)                      # layout_* buffers as asked
+        assert mod.layout_csr_crow.shape[-1] == 1024 // bm + 1
+        if bs < 64:
+            assert mod.mask_tile == 64 and mod.exact_tile == bs
+        elif (bm, bn) != (bs, bs):
+            assert mod.exact_tile == 64 and mod.exact_csr_crow.shape[-1] == 1024 // 64 + 1
+    # row 1 of the merged pair (0, 1) holds column 0... so does row 0: same; row 3 holds column 1, row 2 does not
+    pat = torch.tensor([[[1, 0, 0, 0], [1, 1, 0, 0], [0, 0, 1, 0], [0, 1, 1, 1]]], dtype=torch.uint8)
+    assert not U.tile_sizes_keep_pattern(64, pat, 128, 64, True)
+    assert U.tile_sizes_keep_pattern(64, pat, 64, 32, True)                 # splitting alone never changes it
+    mod = SparseAttention(64, pat, block_m=128)
+    assert mod.exact_tile is None and mod.mask_tile is None and mod.kernel_tile is None
+    # brute force on random causal patterns: expand the merged table and compare
+    rng = np.random.default_rng(3)
+    for _ in range(40):
+        mm = int(rng.choice([2, 4]))
+        n = mm * int(rng.integers(1, 5))  # the builder takes whole merged tiles only
+        dense = np.tril(rng.random((1, n, n)) < 0.5).astype(np.uint8)
+        dense[0, np.arange(n), np.arange(n)] = 1
+        crow, col = U.merge_split_fwd_kernel_blocks(16, torch.from_numpy(dense), 16 * mm, 16)
+        crow, col = crow.numpy().reshape(1, -1), col.numpy().reshape(1, -1, 2)
+        eff = np.zeros_like(dense)
+        for i in range(crow.shape[1] - 1):
+            for c, micro in col[0, crow[0, i]:crow[0, i + 1]]:
+                for s in range(mm):
+                    if i * mm + s < n and s * 16 < micro:
+                        eff[0, i * mm + s, c] = 1
+        same = bool((np.tril(eff) == dense).all())
+        assert U.tile_sizes_keep_pattern(16, torch.from_numpy(dense), 16 * mm, 16, True) == same
 
 
 def test_cpu_tensors_are_refused_loudly():

@@ -344,6 +344,27 @@ def test_paged_decode(page_size, bs, D, head_major):
         assert_close(f"LSE[{i}]", lse[i], rl, atol=LSE_TOL, rtol=0)
 
 
+def test_paged_decode_empty_context_gives_zero_output():
+    """A sequence without any key (context length 0, e.g. a free slot of a serving batch): O = 0,
+    LSE = -inf, and its page-table row is not read."""
+    B, Hq, Hkv, D, Lmax, page = 3, 8, 2, 128, 256, 16
+    g = torch.Generator().manual_seed(20)
+    q = torch.randn(B, Hq, D, generator=g).to(torch.bfloat16).to(DEV)
+    k_pool = torch.randn(4, page, Hkv, D, generator=g).to(torch.bfloat16).to(DEV)
+    v_pool = torch.randn(4, page, Hkv, D, generator=g).to(torch.bfloat16).to(DEV)
+    table = torch.full((B, Lmax // page), -1, dtype=torch.int32, device=DEV)
+    table[1, 0] = 2
+    lens = torch.tensor([0, 5, 0], dtype=torch.int32, device=DEV)
+    mod = _module(Hq, Lmax, 64, 2, 4, num_kv_heads=Hkv)
+    out, lse = mod.paged_decode(q, k_pool, v_pool, table, lens, 0.1, return_lse=True)
+    assert torch.count_nonzero(out[0]) == 0 and torch.count_nonzero(out[2]) == 0
+    assert torch.isneginf(lse[0]).all() and torch.isneginf(lse[2]).all()
+    ro, rl = _seq_oracle(q[1:2].cpu(), k_pool[2, :5].cpu(), v_pool[2, :5].cpu(),
+                         _block_mask(Hq, Lmax, 64, 2, 4, num_kv_heads=Hkv), 64, 0.1)
+    assert_close("O[1]", out[1:2], ro, **TOL)
+    assert_close("LSE[1]", lse[1], rl, atol=LSE_TOL, rtol=0)
+
+
 def test_paged_decode_negative_table_entry_reads_page_zero():
     """A page-table slot marked unused (-1) inside a sequence is a caller's mistake; the kernel
     reads page 0 for it instead of an address before the pools."""

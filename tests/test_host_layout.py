@@ -263,6 +263,114 @@ def test_tile_sizes_given_by_the_caller_keep_the_pattern_or_not():
         assert U.tile_sizes_keep_pattern(16, torch.from_numpy(dense), 16 * mm, 16, True) == same
 
 
+def _fake_fwd_args(B=2, Hq=8, Hkv=2, D=128, Lq=1, Lk=2048, dtype=0, max_row=10):
+    """dk_fwd_args over made-up (never dereferenced) device addresses: a decode-shaped call."""
+    a = _lib.FwdArgs()
+    fake = 0x10000
+
+    def tensor(L, H):
+        return _lib.Tensor(fake, L * H * D, D, H * D)
+    a.q, a.k, a.v, a.o = tensor(Lq, Hq), tensor(Lk, Hkv), tensor(Lk, Hkv), tensor(Lq, Hq)
+    a.lse = _lib.RowVec(None, 0, 0, 0)
+    a.csr = _lib.Lut(fake, fake, Lk // 64 + 1, 1024, 1, Hkv, Lk // 64, 64, 64, 1, max_row, 0)
+    a.seqs = _lib.Seqs(B, Lq, Lk, 0, fake, fake, fake, fake)
+    a.num_q_heads, a.num_kv_heads, a.head_dim = Hq, Hkv, D
+    a.dtype, a.causal, a.impl, a.sm_scale = dtype, 1, 0, 0.1
+    return a
+
+
+def test_c_abi_argument_checks_fail_before_any_launch():
+    """Every entry point validates its arguments on the host and returns a negative code with a
+    message before anything touches the GPU; the workspace queries are pure host functions."""
+    lib = _lib.lib()
+    INVALID = -1
+
+    def refused(rc, text):
+        assert rc == INVALID, rc
+        assert text in lib.dk_last_error().decode(), lib.dk_last_error().decode()
+
+    refused(lib.dk_fwd(None), "args is NULL")
+    a = _fake_fwd_args(Hq=8, Hkv=3)
+    refused(lib.dk_fwd(ctypes.byref(a)), "must be a multiple of num_kv_heads")
+    a = _fake_fwd_args(D=264)
+    refused(lib.dk_fwd(ctypes.byref(a)), "head_dim 264")
+    a = _fake_fwd_args(dtype=7)
+    refused(lib.dk_fwd(ctypes.byref(a)), "unknown dtype")
+    a = _fake_fwd_args()
+    a.csr.num_heads = 5
+    refused(lib.dk_fwd(ctypes.byref(a)), "number of heads in the sparse pattern is 5")
+    a = _fake_fwd_args()
+    a.csr.block_cols = 48
+    refused(lib.dk_fwd(ctypes.byref(a)), "powers of 2")
+    a = _fake_fwd_args()
+    a.csr.sub_block = 8
+    refused(lib.dk_fwd(ctypes.byref(a)), "sub_block must be 0, or 16 / 32")
+    a = _fake_fwd_args()
+    a.seqs.max_k_len = 4096
+    refused(lib.dk_fwd(ctypes.byref(a)), "larger than the maximum length")
+    a = _fake_fwd_args()
+    a.seqs.k_ends = None
+    refused(lib.dk_fwd(ctypes.byref(a)), "must be given together")
+    a = _fake_fwd_args()
+    a.q.ptr = None
+    refused(lib.dk_fwd(ctypes.byref(a)), "q/k/v/o is NULL")
+    # nothing to do is not an error, whatever the pointers are
+    a = _fake_fwd_args(B=0)
+    a.q.ptr = None
+    assert lib.dk_fwd(ctypes.byref(a)) == 0
+
+    # paged decode
+    a = _fake_fwd_args()
+    pg = _lib.PagedKV(0x10000, 128, 16 * 2 * 128, 16 * 2 * 128, 16, 0, 1.0, 1.0)
+    refused(lib.dk_fwd_paged(ctypes.byref(a), None), "page table is NULL")
+    pg.page_size = 24
+    refused(lib.dk_fwd_paged(ctypes.byref(a), ctypes.byref(pg)), "power of two >= 16, got 24")
+    pg.page_size, pg.kv_dtype = 16, 1
+    refused(lib.dk_fwd_paged(ctypes.byref(a), ctypes.byref(pg)), "kv_dtype must be the q dtype")
+    pg.kv_dtype, pg.k_scale = _lib.DK_FP8_E4M3, 0.0
+    refused(lib.dk_fwd_paged(ctypes.byref(a), ctypes.byref(pg)), "scales must be positive")
+    pg.kv_dtype, pg.k_scale = 0, 1.0
+    refused(lib.dk_fwd_paged(ctypes.byref(a), ctypes.byref(pg)), "decode workspace too small")
+    a.seqs.q_starts = a.seqs.q_ends = a.seqs.k_starts = a.seqs.k_ends = None
+    a.seqs.max_q_len = a.seqs.max_k_len
+    refused(lib.dk_fwd_paged(ctypes.byref(a), ctypes.byref(pg)), "per-sequence lengths")
+
+    # workspace queries: decode-shaped calls ask for [batch][q heads][units][D + 2] floats
+    a = _fake_fwd_args(B=2, Hq=8, Hkv=2, D=128, max_row=10)
+    need = lib.dk_fwd_workspace_bytes(ctypes.byref(a))
+    assert need > 0 and need % (2 * 8 * 130 * 4) == 0 and need // (2 * 8 * 130 * 4) >= 4
+    a.seqs.max_q_len = 7                       # neither decode nor prefill of the same length
+    assert lib.dk_fwd_workspace_bytes(ctypes.byref(a)) == 0
+    a = _fake_fwd_args(D=160)                  # no matrix-core decode kernel for this head_dim
+    assert lib.dk_fwd_workspace_bytes(ctypes.byref(a)) == 0
+
+    # backward: paddings are refused as in the reference; GQA asks for fp32 per-head partials
+    b = _lib.BwdArgs()
+    t = _lib.Tensor(0x10000, 1024 * 8 * 128, 128, 8 * 128)
+    tk = _lib.Tensor(0x10000, 1024 * 2 * 128, 128, 2 * 128)
+    b.q, b.o, b.dout, b.dq = t, t, t, t
+    b.k, b.v, b.dk, b.dv = tk, tk, tk, tk
+    b.lse = _lib.RowVec(0x10000, 8 * 1024, 1024, 1)
+    b.dlse = _lib.RowVec(None, 0, 0, 0)
+    b.delta = 0x10000
+    b.csr = _lib.Lut(0x10000, 0x10000, 17, 1024, 1, 2, 16, 64, 64, 1, 0, 0)
+    b.csc = _lib.Lut(0x10000, 0x10000, 17, 1024, 1, 2, 16, 64, 64, 1, 0, 0)
+    b.seqs = _lib.Seqs(3, 1024, 1024, 0, None, None, None, None)
+    b.num_q_heads, b.num_kv_heads, b.head_dim, b.dtype, b.causal, b.impl, b.sm_scale = 8, 2, 128, 0, 1, 0, 0.1
+    assert lib.dk_bwd_workspace_bytes(ctypes.byref(b)) == 2 * 3 * 8 * 1024 * 128 * 4
+    b.num_kv_heads = 8
+    b.csr.num_heads = b.csc.num_heads = 8
+    assert lib.dk_bwd_workspace_bytes(ctypes.byref(b)) == 0
+    b.seqs = _lib.Seqs(3, 1024, 1024, 0, 0x10000, 0x10000, 0x10000, 0x10000)
+    refused(lib.dk_bwd(ctypes.byref(b)), "does not support paddings")
+    b.seqs = _lib.Seqs(3, 1024, 1024, 0, None, None, None, None)
+    b.csc.entry_width = 2
+    refused(lib.dk_bwd(ctypes.byref(b)), "csc table cannot carry values")
+    b.csc.entry_width = 1
+    b.delta = None
+    refused(lib.dk_bwd(ctypes.byref(b)), "lse / delta is NULL")
+
+
 def test_cpu_tensors_are_refused_loudly():
     m = LocalStrideSparseAttention(2, 128, 64, 1, 2)
     x = torch.zeros(1, 128, 2, 64)

@@ -12,7 +12,8 @@ namespace dk {
 int launch_generic_fwd(const FwdParams &p, int dtype, hipStream_t stream);
 int launch_generic_bwd(const BwdParams &p, int dtype, hipStream_t stream);
 bool mfma_fwd_supported(const FwdParams &p, int dtype);
-int launch_mfma_fwd(const FwdParams &p, int dtype, hipStream_t stream);
+int launch_mfma_fwd(const FwdParams &p, int dtype, void *workspace, size_t workspace_bytes, hipStream_t stream);
+size_t mfma_fwd_workspace_bytes(const FwdParams &p);
 bool mfma_bwd_supported(const BwdParams &p, int dtype);
 int launch_mfma_bwd(const BwdParams &p, int dtype, void *workspace, size_t workspace_bytes, hipStream_t stream);
 size_t mfma_bwd_workspace_bytes(const BwdParams &p);
@@ -159,6 +160,7 @@ size_t dk_fwd_workspace_bytes(const dk_fwd_args *a) {
   FwdParams p;
   if (make_fwd_params(a, p) != DK_OK) return 0;
   if (a->impl != DK_IMPL_GENERIC && decode_supported(p, a->dtype)) return decode_workspace_bytes(p);
+  if (a->impl != DK_IMPL_GENERIC && mfma_fwd_supported(p, a->dtype)) return mfma_fwd_workspace_bytes(p);
   return 0;
 }
 
@@ -173,7 +175,8 @@ int dk_fwd(const dk_fwd_args *a) {
     if (decode_supported(p, a->dtype) && a->workspace &&
         a->workspace_bytes >= decode_workspace_bytes(p))
       return launch_decode(p, a->dtype, a->workspace, a->workspace_bytes, stream);
-    if (mfma_fwd_supported(p, a->dtype)) return launch_mfma_fwd(p, a->dtype, stream);
+    if (mfma_fwd_supported(p, a->dtype))
+      return launch_mfma_fwd(p, a->dtype, a->workspace, a->workspace_bytes, stream);
     if (a->impl == DK_IMPL_MFMA)
       return fail(DK_ERR_UNSUPPORTED, "no MFMA forward kernel for dtype %d, head_dim %d, tiles (%d, %d)", a->dtype,
                   p.D, p.csr.block_rows, p.csr.block_cols);

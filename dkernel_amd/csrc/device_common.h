@@ -55,6 +55,9 @@ struct LutView {
 struct SeqView {
   int32_t batch, max_q_len, max_k_len, packed;
   const int32_t *q_starts, *q_ends, *k_starts, *k_ends;
+  // packed inputs, optional: batch + 1 ints, entry b = work items (q tiles or pairs of q tiles) of
+  // the sequences before b, written by a small kernel ahead of the one that reads it
+  int32_t *item_offsets = nullptr;
 };
 
 // Paged K/V (decode only): k / v point at page pools, token t of sequence b lives in page
@@ -103,7 +106,8 @@ struct SeqInfo {
   int q_start, q_len, k_start, k_len, past;
 };
 
-__device__ __forceinline__ SeqInfo load_seq(const SeqView &s, int b, int causal) {
+// Geometry of sequence b as this lane sees it (b may differ between lanes).
+__device__ __forceinline__ SeqInfo load_seq_lane(const SeqView &s, int b, int causal) {
   SeqInfo r;
   r.b = b;
   if (s.q_starts) {
@@ -122,6 +126,12 @@ __device__ __forceinline__ SeqInfo load_seq(const SeqView &s, int b, int causal)
   if (r.k_len < 0) r.k_len = 0;
   r.past = causal ? r.k_len - r.q_len : 0;
   if (r.past < 0) r.past = 0;
+  return r;
+}
+
+// The same for a b that every lane of the wave shares.
+__device__ __forceinline__ SeqInfo load_seq(const SeqView &s, int b, int causal) {
+  SeqInfo r = load_seq_lane(s, b, causal);
   // b is the same for every lane of a wave, so the fields are too; saying so keeps the
   // addresses derived from them in scalar registers
   r.q_start = __builtin_amdgcn_readfirstlane(r.q_start);
@@ -139,11 +149,122 @@ __device__ __forceinline__ int seq_row_blocks(const SeqInfo &s, int block_rows) 
   return (s.past + s.q_len - 1) / block_rows - s.past / block_rows + 1;
 }
 
-// Maps (blockIdx.x = tile index, blockIdx.z = batch) to a sequence and the
-// index of the tile within it; tiles_per_block sub-tiles per row block.
-// Returns false when the workgroup has nothing to do.  For packed inputs
-// the sequences are scanned on the device (batch is small), so no tile map
-// has to be built on the host.
+// Pairs of adjacent table rows (2u, 2u + 1) that hold queries of a sequence.
+__device__ __forceinline__ int seq_row_pairs(const SeqInfo &s) {
+  if (s.q_len <= 0) return 0;
+  const int first = s.past / 64, last = (s.past + s.q_len - 1) / 64;
+  return (last >> 1) - (first >> 1) + 1;
+}
+
+// Packed inputs: the sequences share one token dimension and work items (q tiles, pairs of q
+// tiles) are numbered through all of them, count(sequence) items each.  Finds the sequence that
+// holds `item` and the item's index inside it; returns -1 beyond the last item.  The search runs
+// on the device (no host copy of the lengths), a wave at a time with every lane active and the
+// same `item`: each lane adds up the counts of batch / 64 consecutive sequences, a prefix sum over
+// the lanes names the lane whose chunk holds the item, and its sequences are searched the same
+// way, 64 at a time -- a few dependent loads whatever the batch size.
+template <typename Count>
+__device__ __forceinline__ int find_packed_sequence(const SeqView &s, int causal, int item, Count count,
+                                                    int &index_in_seq) {
+  if (s.item_offsets) {
+    // the running item counts are there: bisect (wave-uniform addresses; zero-item sequences
+    // share their successor's offset and are never the answer)
+    const int32_t *off = s.item_offsets;
+    if (item >= __builtin_amdgcn_readfirstlane(off[s.batch])) return -1;
+    int lo = 0, hi = s.batch;  // off[lo] <= item < off[hi]
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (__builtin_amdgcn_readfirstlane(off[mid]) <= item)
+        lo = mid;
+      else
+        hi = mid;
+    }
+    index_in_seq = item - __builtin_amdgcn_readfirstlane(off[lo]);
+    return lo;
+  }
+  const int lane = threadIdx.x & 63;
+  const int per_lane = (s.batch + 63) / 64;
+  int mine = 0;
+  // (indices clamped instead of branched around, eight at a time: the loads of a group are
+  // independent and leave together)
+  for (int i0 = 0; i0 < per_lane; i0 += 8) {
+    int n[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int b = lane * per_lane + i0 + i;
+      const bool real = i0 + i < per_lane && b < s.batch;
+      n[i] = count(load_seq_lane(s, real ? b : 0, causal));
+      if (!real) n[i] = 0;
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) mine += n[i];
+  }
+  auto prefix = [&](int v) {  // inclusive sum over the lanes
+    for (int off = 1; off < 64; off <<= 1) {
+      const int t = __shfl_up(v, off);
+      if (lane >= off) v += t;
+    }
+    return v;
+  };
+  const int upto = prefix(mine);
+  const unsigned long long holders = __ballot(item < upto);
+  if (holders == 0) return -1;
+  const int owner = __ffsll(holders) - 1;                     // first lane whose chunk reaches past the item
+  int before = __shfl(upto - mine, owner);                    // items of the chunks before it
+  if (per_lane == 1) {
+    index_in_seq = __builtin_amdgcn_readfirstlane(item - before);
+    return __builtin_amdgcn_readfirstlane(owner);
+  }
+  for (int j0 = 0; j0 < per_lane; j0 += 64) {
+    const int j = j0 + lane, b = owner * per_lane + j;
+    const int n = (j < per_lane && b < s.batch) ? count(load_seq_lane(s, b, causal)) : 0;
+    const int upto2 = prefix(n);
+    const unsigned long long hit = __ballot(item < before + upto2);
+    if (hit != 0) {
+      const int l2 = __ffsll(hit) - 1;
+      index_in_seq = __builtin_amdgcn_readfirstlane(item - before - __shfl(upto2 - n, l2));
+      return __builtin_amdgcn_readfirstlane(owner * per_lane + j0 + l2);
+    }
+    before += __shfl(upto2, 63);
+  }
+  return -1;  // not reached: the owner's chunk holds the item
+}
+
+// Fills SeqView::item_offsets: one workgroup of 1024 threads; count(sequence) as in
+// find_packed_sequence.  Thread t adds up batch / 1024 consecutive sequences, the partial sums
+// are scanned in LDS, and each thread writes the running counts of its sequences.
+template <typename Count>
+__device__ __forceinline__ void write_item_offsets(const SeqView &s, int causal, Count count, int32_t *out) {
+  __shared__ int part[1024];
+  const int t = threadIdx.x;
+  const int per = (s.batch + 1023) / 1024;
+  int sum = 0;
+  for (int i = 0; i < per; ++i) {
+    const int b = t * per + i;
+    if (b < s.batch) sum += count(load_seq_lane(s, b, causal));
+  }
+  part[t] = sum;
+  __syncthreads();
+  for (int off = 1; off < 1024; off <<= 1) {
+    const int v = t >= off ? part[t - off] : 0;
+    __syncthreads();
+    part[t] += v;
+    __syncthreads();
+  }
+  int run = part[t] - sum;
+  for (int i = 0; i < per; ++i) {
+    const int b = t * per + i;
+    if (b < s.batch) {
+      out[b] = run;
+      run += count(load_seq_lane(s, b, causal));
+    }
+  }
+  if (t == 1023) out[s.batch] = part[1023];
+}
+
+// Maps (tile_x = tile index, bz = batch index) to a sequence and the index of the tile within
+// it; tiles_per_block sub-tiles per row block.  Returns false when the workgroup has nothing to
+// do.  Packed inputs: tile_x counts through all sequences (every lane of the wave must call).
 __device__ __forceinline__ bool resolve_tile(const SeqView &s, int causal, int block_rows,
                                              int tiles_per_block, int tile_x, int bz, SeqInfo &info,
                                              int &tile_in_seq) {
@@ -152,18 +273,12 @@ __device__ __forceinline__ bool resolve_tile(const SeqView &s, int causal, int b
     tile_in_seq = tile_x;
     return tile_x < seq_row_blocks(info, block_rows) * tiles_per_block;
   }
-  int acc = 0;
-  for (int b = 0; b < s.batch; ++b) {
-    SeqInfo t = load_seq(s, b, causal);
-    int n = seq_row_blocks(t, block_rows) * tiles_per_block;
-    if (tile_x < acc + n) {
-      info = t;
-      tile_in_seq = tile_x - acc;
-      return true;
-    }
-    acc += n;
-  }
-  return false;
+  const int b = find_packed_sequence(
+      s, causal, tile_x, [&](const SeqInfo &t) { return seq_row_blocks(t, block_rows) * tiles_per_block; },
+      tile_in_seq);
+  if (b < 0) return false;
+  info = load_seq(s, b, causal);
+  return true;
 }
 
 }  // namespace dk

@@ -63,22 +63,16 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
     // workgroup = table rows 2u and 2u + 1 of one head (one per wave pair); tiles_y counts pairs
     int u;
     if (p.seqs.packed) {
-      // the sequences share one token dimension: blockIdx.y counts row pairs over all of them
-      // (the sequences are scanned on the device, as in resolve_tile)
-      int acc = 0, found = 0;
-      for (int b = 0; b < p.seqs.batch && !found; ++b) {
-        const SeqInfo t = load_seq(p.seqs, b, p.causal);
-        if (t.q_len <= 0) continue;
-        const int f = t.past / 64, l = (t.past + t.q_len - 1) / 64;
-        const int n = (l >> 1) - (f >> 1) + 1;
-        if ((int)blockIdx.y < acc + n) {
-          sq = t, first_rb = f, last_rb = l;
-          u = (f >> 1) + (int)blockIdx.y - acc;
-          found = 1;
-        }
-        acc += n;
-      }
-      if (!found) return;
+      // the sequences share one token dimension: row pairs are counted through all of them (last
+      // pair first: within a sequence the longest rows start first, as for unpacked inputs)
+      int idx;
+      const int b = find_packed_sequence(
+          p.seqs, p.causal, tiles_y - 1 - (int)blockIdx.y,
+          [](const SeqInfo &t) { return seq_row_pairs(t); }, idx);
+      if (b < 0) return;
+      sq = load_seq(p.seqs, b, p.causal);
+      first_rb = sq.past / 64, last_rb = (sq.past + sq.q_len - 1) / 64;
+      u = (first_rb >> 1) + idx;
     } else {
       sq = load_seq(p.seqs, blockIdx.z, p.causal);
       if (sq.q_len <= 0) return;
@@ -89,7 +83,7 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
     rb = 2 * u + (wave >> 1);
     tile = rb - first_rb;  // outside [0, last_rb - first_rb]: this wave pair has no rows (row_ok false everywhere)
   } else {
-    const int ty = p.seqs.packed ? blockIdx.y : tiles_y - 1 - (int)blockIdx.y;
+    const int ty = tiles_y - 1 - (int)blockIdx.y;  // longest rows first
     if (!resolve_tile(p.seqs, p.causal, 64, 1, ty, blockIdx.z, sq, tile)) return;
     rb = sq.past / 64 + tile;
   }
@@ -399,7 +393,7 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
 
   SeqInfo sq;
   int tile;
-  const int ty = p.seqs.packed ? blockIdx.y : tiles_y - 1 - (int)blockIdx.y;
+  const int ty = tiles_y - 1 - (int)blockIdx.y;  // longest rows first
   if (!resolve_tile(p.seqs, p.causal, 64, 1, ty, blockIdx.z, sq, tile)) return;
   const int rb = sq.past / 64 + tile;
   const int tid = threadIdx.x, lane = tid & 63;
@@ -680,6 +674,32 @@ static int fwd_group(const FwdParams &p) {
   return 1;
 }
 
+// Packed inputs: running work-item counts of the sequences (q tiles, or pairs of q tiles for the
+// row-pair kernel), so that a workgroup finds its sequence by bisection instead of adding up the
+// sequences before it.
+__global__ __launch_bounds__(1024) void packed_item_offsets_kernel(const SeqView s, int causal, int pairs,
+                                                                   int32_t *out) {
+  if (pairs)
+    write_item_offsets(s, causal, [](const SeqInfo &t) { return seq_row_pairs(t); }, out);
+  else
+    write_item_offsets(s, causal, [](const SeqInfo &t) { return seq_row_blocks(t, 64); }, out);
+}
+
+static int launch_item_offsets(const FwdParams &p, bool pairs, hipStream_t stream) {
+  if (!p.seqs.packed || !p.seqs.item_offsets) return DK_OK;
+  SeqView s = p.seqs;
+  s.item_offsets = nullptr;
+  hipLaunchKernelGGL(packed_item_offsets_kernel, dim3(1), dim3(1024), 0, stream, s, p.causal, pairs ? 1 : 0,
+                     p.seqs.item_offsets);
+  DK_HIP_CHECK(hipGetLastError());
+  return DK_OK;
+}
+
+// Scratch the forward can use: batch + 1 ints for packed inputs.
+size_t mfma_fwd_workspace_bytes(const FwdParams &p) {
+  return p.seqs.packed ? (((size_t)p.seqs.batch + 1) * sizeof(int32_t) + 15) / 16 * 16 : 0;
+}
+
 bool mfma_fwd_supported(const FwdParams &p, int dtype) {
   return (dtype == DK_BF16 || dtype == DK_F16) && mfma_head_dim_ok(p.D) && p.csr.block_rows == 64 &&
          p.csr.block_cols == 64 && p.vec_ok &&
@@ -691,6 +711,7 @@ static int launch_tdg(const FwdParams &p, dim3 grid, int tiles_y, hipStream_t st
   constexpr int smem = 2 * FwdSmem<D>::kStage;
   DK_ALLOW_DYNAMIC_LDS((mfma_fwd_kernel<T, D, G, PAD, false>), smem);
   grid.x = p.Hq / G;
+  if (int rc = launch_item_offsets(p, false, stream)) return rc;
   // One head per workgroup and one q tile (row pairs switched off): one wave per SIMD, where
   // the software-pipelined kernel is the faster one.  With two waves per SIMD it is not: it
   // needs more registers than the 256 a wave gets, and spilled loader state is reloaded
@@ -727,6 +748,7 @@ static int launch_row_pairs(const FwdParams &p, hipStream_t stream) {
     pairs = (((past + s.max_q_len - 1) / 64) >> 1) - ((past / 64) >> 1) + 1;
   }
   DK_REQUIRE(pairs <= 65535, "too many q tiles for one launch (%d)", pairs);
+  if (int rc = launch_item_offsets(p, true, stream)) return rc;
   hipLaunchKernelGGL((mfma_fwd_kernel<T, D, 2, PAD, true>), dim3(p.Hq, pairs, s.packed ? 1 : s.batch), dim3(256), smem,
                      stream, p, pairs);
   DK_HIP_CHECK(hipGetLastError());
@@ -753,6 +775,7 @@ static int launch_sub_g(const FwdParams &p, dim3 grid, int tiles_y, hipStream_t 
   constexpr int smem = 2 * FwdSmem<D>::kStage;
   DK_ALLOW_DYNAMIC_LDS((mfma_fwd_kernel<T, D, G, PAD, false, true>), smem);
   grid.x = p.Hq / G;
+  if (int rc = launch_item_offsets(p, false, stream)) return rc;
   hipLaunchKernelGGL((mfma_fwd_kernel<T, D, G, PAD, false, true>), grid, dim3(128 * G), smem, stream, p, tiles_y);
   DK_HIP_CHECK(hipGetLastError());
   return DK_OK;
@@ -781,7 +804,10 @@ static int launch_t(const FwdParams &p, dim3 grid, int tiles_y, hipStream_t stre
   return p.D > 64 ? launch_tdp<T, 128, true>(p, grid, tiles_y, stream) : launch_tdp<T, 64, true>(p, grid, tiles_y, stream);
 }
 
-int launch_mfma_fwd(const FwdParams &p, int dtype, hipStream_t stream) {
+int launch_mfma_fwd(const FwdParams &p_in, int dtype, void *workspace, size_t workspace_bytes, hipStream_t stream) {
+  FwdParams p = p_in;
+  if (p.seqs.packed && workspace && workspace_bytes >= mfma_fwd_workspace_bytes(p) && ((uintptr_t)workspace % 4) == 0)
+    p.seqs.item_offsets = (int32_t *)workspace;
   const SeqView &s = p.seqs;
   int tiles;
   if (s.packed)

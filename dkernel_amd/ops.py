@@ -28,6 +28,7 @@ _impl = _lib.DK_IMPL_AUTO
 
 
 _bwd_workspace = True  # hand dk_bwd the scratch it asks for (off: tests of the path without it)
+_fwd_workspace = True  # the same for dk_fwd
 
 
 def set_impl(name: str) -> None:
@@ -127,7 +128,7 @@ last_fwd_workspace_bytes = 0  # scratch the library asked for in the latest forw
 def _run_fwd(args: _lib.FwdArgs, device) -> None:
     global last_fwd_workspace_bytes
     lib = _lib.lib()
-    need = lib.dk_fwd_workspace_bytes(C.byref(args))
+    need = lib.dk_fwd_workspace_bytes(C.byref(args)) if _fwd_workspace else 0
     last_fwd_workspace_bytes = need
     ws = None
     if need:

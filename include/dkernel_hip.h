@@ -152,13 +152,16 @@ typedef struct dk_fwd_args {
   int32_t causal;
   int32_t impl;   /* enum dk_impl */
   float sm_scale;
-  void *workspace;        /* device scratch for split-KV decode, may be NULL */
+  void *workspace;        /* optional device scratch (16-byte aligned): split-KV decode partials,
+                             or the running tile counts of packed sequences; may be NULL */
   size_t workspace_bytes;
   void *stream;           /* hipStream_t */
 } dk_fwd_args;
 
 int dk_fwd(const dk_fwd_args *args);
-/* Scratch that dk_fwd can use for these arguments (0 = none needed). */
+/* Scratch that dk_fwd can use for these arguments (0 = none needed): single-token decode runs
+ * the split-KV kernels only with it; packed prefill runs without it too, but then every
+ * workgroup scans the sequence lengths to find its own, which costs with hundreds of sequences. */
 size_t dk_fwd_workspace_bytes(const dk_fwd_args *args);
 
 /* Paged K/V cache for single-token decode (serving).  args->k / args->v point at

@@ -488,6 +488,43 @@ def test_packed_varlen_prefill_and_decode(impl, D, bs):
                      atol=1e-2, rtol=1e-2)
 
 
+@pytest.mark.parametrize("Hq,Hkv,nseq", [(4, 2, 200), (2, 2, 700)])
+def test_packed_prefill_with_hundreds_of_sequences(monkeypatch, Hq, Hkv, nseq):
+    """A workgroup finds its sequence by bisecting running tile counts that a small kernel wrote
+    into the scratch, or, without scratch, by a wave-wide scan of the lengths: both must place
+    every tile (sequences of 0 to 150 tokens, several lanes' worth of them), agree bit for bit,
+    and match the generic kernels and the oracle."""
+    D, bs = 64, 64
+    sm = 1 / math.sqrt(D)
+    rng = np.random.default_rng(nseq)
+    lens = [int(x) for x in rng.integers(0, 151, nseq)]
+    lens[3] = lens[nseq // 2] = lens[-1] = 0
+    T = sum(lens)
+    g = torch.Generator().manual_seed(20)
+    q, k, v = (torch.randn(T, h, D, generator=g).to(torch.bfloat16) for h in (Hq, Hkv, Hkv))
+    cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32)
+    mod = _module(Hq, 256, bs, 2, 2, num_kv_heads=Hkv)
+    bm = _block_mask(Hq, 256, bs, 2, 2, num_kv_heads=Hkv)
+    res = {}
+    for name, impl_name, ws in (("bisect", "mfma", True), ("scan", "mfma", False), ("generic", "generic", True)):
+        ops.set_impl(impl_name)
+        monkeypatch.setattr(ops, "_fwd_workspace", ws)
+        try:
+            res[name] = mod(q.to(DEV), k.to(DEV), v.to(DEV), sm, cu_seqlen_k=cu.to(DEV), return_lse=True)
+            assert (ops.last_fwd_workspace_bytes > 0) == (name == "bisect")
+        finally:
+            ops.set_impl("auto")
+    assert torch.equal(res["bisect"][0], res["scan"][0]) and torch.equal(res["bisect"][1], res["scan"][1])
+    assert_close("O vs generic", res["bisect"][0], res["generic"][0], **TOL)
+    assert_close("LSE vs generic", res["bisect"][1], res["generic"][1], atol=LSE_TOL, rtol=0)
+    for i in list(range(0, nseq, 37)) + [nseq - 2]:
+        s, e = int(cu[i]), int(cu[i + 1])
+        if e > s:
+            ro, rl = _seq_oracle(q[s:e], k[s:e], v[s:e], bm, bs, sm)
+            assert_close(f"O[{i}]", res["bisect"][0][s:e], ro, **TOL)
+            assert_close(f"LSE[{i}]", res["bisect"][1][:, s:e], rl, atol=LSE_TOL, rtol=0)
+
+
 def test_packed_chunked_prefill_every_sequence_starts_inside_a_block(impl):
     """Packed chunked prefill where every sequence's queries start inside a row block and end
     in another: each touches ceil(q_len / 64) + 1 row blocks, the most the launch has to cover."""

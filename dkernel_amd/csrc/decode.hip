@@ -133,7 +133,9 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(2, 2))) 
     scalar_load2(p.csr.ptr + lh * p.csr.ptr_sh + rb, p.csr.ptr + lh * p.csr.ptr_sh + rb + 1, row0, row1);
   // the row's entries are split evenly over as many units as the unit size asks for
   const int n_ent = row1 - row0;
-  const int u_cnt = decode_row_units(n_ent, unit_blocks, W);
+  // never more than the host sized the grid and the workspace for: a row longer than the caller's
+  // max_row_entries hint said is still cut into max_units units, each with a larger share
+  const int u_cnt = min(decode_row_units(n_ent, unit_blocks, W), max_units);
   if ((int)blockIdx.x * W >= u_cnt && (blockIdx.x > 0 || W == 1)) return;  // nothing for this workgroup
   const bool merge_here = W > 1 && u_cnt <= W;  // (a row without entries is written here too: O = 0, LSE = -inf)
   const int per = u_cnt > 0 ? (n_ent + u_cnt - 1) / u_cnt : 0;
@@ -166,23 +168,30 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(2, 2))) 
   // page table beyond the sequence's last token are never read; a negative entry inside the
   // sequence (a caller's mistake: such slots mark unused pages) is read as page 0 rather than
   // as an address before the pool.
+  // A unit of more than 16 entries (only when the caller's max_row_entries hint understated the
+  // row) reloads the register every 16 entries.
   int my_page = 0;
-  if constexpr (PAGED) {
-    const int j = lane >> 2, s = lane & 3;
+  auto load_pages = [&](int j0) {  // pages of entries e0 + j0 .. e0 + j0 + 15
+    int pg = 0;
+    const int j = j0 + (lane >> 2), s = lane & 3;
     const int ps = 1 << p.paged.page_shift;
     if (j < e1 - e0) {
       const int col = cols[(e0 + j) * EW];
       const int tok = col * 64 + (ps < 64 ? s * ps : 0);
       if (col >= 0 && tok < sq.k_len && (s == 0 || s * ps < 64))
-        my_page = max(p.paged.table[b * p.paged.table_sb + (tok >> p.paged.page_shift)], 0);
+        pg = max(p.paged.table[b * p.paged.table_sb + (tok >> p.paged.page_shift)], 0);
     }
-  }
+    return pg;
+  };
+  if constexpr (PAGED) my_page = load_pages(0);
 
   // half block hb of this unit = keys cols[e0 + hb/2] * 64 + 32 * (hb & 1) + [0, 32)
   constexpr int HCH = 32 * CPR / 64;  // 16-byte chunks per lane per half tile
   uint4 kreg[HCH], vreg[HCH];
   auto prefetch = [&](int hb, int col, int bits) {
     const int key0 = col * 64 + (hb & 1) * 32;
+    if constexpr (PAGED)
+      if (hb > 0 && (hb & 31) == 0) my_page = load_pages(hb >> 1);  // (never with the default unit sizes)
     if (SUB && half_bits(bits, hb) == 0) return;  // no attended key in this half: neither read nor used
     // element offset of row r of the half block from kbase / vbase
     int pg_lo = 0, pg_hi = 0, in_page0 = 0;
@@ -190,8 +199,8 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(2, 2))) 
       // the half block's 32 keys lie in one page, or in two pages of 16
       const int psl = p.paged.page_shift, half = hb & 1;
       const int s_lo = psl < 6 ? (half * 32) >> psl : 0, s_hi = psl < 6 ? (half * 32 + 16) >> psl : 0;
-      pg_lo = __builtin_amdgcn_readlane(my_page, ((hb >> 1) * 4 + s_lo) & 63);
-      pg_hi = __builtin_amdgcn_readlane(my_page, ((hb >> 1) * 4 + s_hi) & 63);
+      pg_lo = __builtin_amdgcn_readlane(my_page, (((hb >> 1) & 15) * 4 + s_lo) & 63);
+      pg_hi = __builtin_amdgcn_readlane(my_page, (((hb >> 1) & 15) * 4 + s_hi) & 63);
       in_page0 = key0 & ((1 << psl) - 1);
     }
     auto k_off = [&](int r) -> int64_t {
@@ -434,7 +443,7 @@ __global__ __launch_bounds__(64) void decode_combine_kernel(const FwdParams p, c
   if (sq.k_len > 0 && rb < p.csr.num_rows) {
     const int lh = lut_head(p.csr, h, p.Hq, p.Hkv);
     const int n = scalar_load(p.csr.ptr + lh * p.csr.ptr_sh + rb + 1) - scalar_load(p.csr.ptr + lh * p.csr.ptr_sh + rb);
-    units = decode_row_units(n, unit_blocks, merged_units > 0 ? merged_units : 1);
+    units = min(decode_row_units(n, unit_blocks, merged_units > 0 ? merged_units : 1), max_units);  // as the partial kernel
   }
   // rows of at most merged_units units were finished by the partial kernel (merged_units > 0)
   if (merged_units > 0 && units <= merged_units) return;

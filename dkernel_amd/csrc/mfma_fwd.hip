@@ -703,7 +703,8 @@ size_t mfma_fwd_workspace_bytes(const FwdParams &p) {
 bool mfma_fwd_supported(const FwdParams &p, int dtype) {
   return (dtype == DK_BF16 || dtype == DK_F16) && mfma_head_dim_ok(p.D) && p.csr.block_rows == 64 &&
          p.csr.block_cols == 64 && p.vec_ok &&
-         (p.csr.entry_width == 1 || p.csr.sub_block != 0);
+         (p.csr.entry_width == 1 || p.csr.sub_block != 0) &&
+         p.scale_log2 > 0.f;  // the row maximum is taken before scaling (a scale <= 0 runs on the generic kernels)
 }
 
 template <typename T, int D, int G, bool PAD>

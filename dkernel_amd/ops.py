@@ -380,7 +380,8 @@ def varlen_sparse_attn(q: Tensor, k: Tensor, v: Tensor,
                        inference: bool = True,
                        causal: bool = True,
                        return_lse: bool = False,
-                       lut_group: int = 1):
+                       lut_group: int = 1,
+                       lut_max_row: int = 0):
     """Packed variable-length inputs (total_tokens, heads, head_dim) with
     cumulative sequence lengths.  Reference:
     dkernel/ops/sparse_attn_inference.py:150-287.  The query tokens of a
@@ -416,7 +417,7 @@ def varlen_sparse_attn(q: Tensor, k: Tensor, v: Tensor,
     args = _lib.FwdArgs()
     args.q, args.k, args.v, args.o = (_tensor3(x) for x in (q, k, v, out))
     args.lse = _rowvec(lse, (0, lse.stride(0), lse.stride(1))) if lse is not None else _rowvec(None)
-    args.csr = _lut(sparse_layout, dev, lut_group)
+    args.csr = _lut(sparse_layout, dev, lut_group, lut_max_row)
     isz = cu_q.element_size()
     args.seqs = _lib.Seqs(batch_size, q.size(0), k.size(0), 3 if single_query else 1,
                           cu_q.data_ptr(), cu_q.data_ptr() + isz, cu_k.data_ptr(), cu_k.data_ptr() + isz)
@@ -494,7 +495,7 @@ class _sparse_attention(torch.autograd.Function):
             ctx.message = "Currently does not suppoort variable length inputs. WIP."
             res = varlen_sparse_attn(q, k, v, inf_kwargs["cu_seqlen_k"], inf_kwargs.get("cu_seqlen_q", None),
                                      sm_scale, layout_csr, max_seqlen=max_seqlen, causal=causal,
-                                     return_lse=return_lse, lut_group=lut_group)
+                                     return_lse=return_lse, lut_group=lut_group, lut_max_row=lut_max_row)
             output, lse = res if return_lse else (res, None)
         else:
             assert k.size(seq_dim) <= max_seqlen, \

@@ -15,6 +15,7 @@ LIB_PATH = os.environ.get("DKERNEL_AMD_LIB") or os.path.join(_HERE, "libdkernel_
 DK_BF16, DK_F16, DK_F32, DK_FP8_E4M3 = 0, 1, 2, 3
 DK_IMPL_AUTO, DK_IMPL_GENERIC, DK_IMPL_MFMA = 0, 1, 2
 DK_ERR_INVALID, DK_ERR_UNSUPPORTED, DK_ERR_HIP = -1, -2, -3
+DK_NOALLOC_SCRATCH_BYTES = 8 << 20
 
 i32, i64, f32, vp = C.c_int32, C.c_int64, C.c_float, C.c_void_p
 
@@ -74,6 +75,7 @@ SYMBOLS = {
     "dk_kv_cache_efficient": (C.c_int, [vp, i32, i32, i32, i32, i32]),
     "dk_fwd": (C.c_int, [C.POINTER(FwdArgs)]),
     "dk_fwd_workspace_bytes": (C.c_size_t, [C.POINTER(FwdArgs)]),
+    "dk_fwd_noalloc": (C.c_int, [C.POINTER(FwdArgs)]),
     "dk_fwd_paged": (C.c_int, [C.POINTER(FwdArgs), C.POINTER(PagedKV)]),
     "dk_bwd": (C.c_int, [C.POINTER(BwdArgs)]),
     "dk_bwd_workspace_bytes": (C.c_size_t, [C.POINTER(BwdArgs)]),

@@ -150,11 +150,55 @@ static int make_bwd_params(const dk_bwd_args *a, BwdParams &p, bool &empty) {
   return DK_OK;
 }
 
+// ---------------------------------------------------------------------------
+// Scratch of dk_fwd_noalloc: a file-scope device array, so that callers that may not allocate
+// (HIP graph capture, serving loops) need no workspace of their own.  Every GPU the library runs
+// on holds its own copy at its own address; the array's name is only a host-side handle, so the
+// device address is looked up once per device and that pointer is what kernels receive.
+// ---------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[DK_NOALLOC_SCRATCH_BYTES];
+
+static int static_scratch(void **out) {
+  constexpr int kMaxDevices = 64;
+  static std::atomic<void *> per_device[kMaxDevices];  // zero-initialised
+  int dev = 0;
+  DK_HIP_CHECK(hipGetDevice(&dev));
+  DK_REQUIRE(dev >= 0 && dev < kMaxDevices, "device ordinal %d beyond %d", dev, kMaxDevices);
+  void *ptr = per_device[dev].load(std::memory_order_acquire);
+  if (!ptr) {  // first call on this device (a race between threads only repeats the lookup)
+    DK_HIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    DK_REQUIRE(ptr != nullptr, "no device address for the static scratch");
+    per_device[dev].store(ptr, std::memory_order_release);
+  }
+  *out = ptr;
+  return DK_OK;
+}
+
 }  // namespace dk
 
 using namespace dk;
 
 extern "C" {
+
+int dk_fwd_noalloc(const dk_fwd_args *a) {
+  clear_error();
+  DK_REQUIRE(a != nullptr, "args is NULL");
+  dk_fwd_args b = *a;
+  b.workspace = nullptr;
+  b.workspace_bytes = 0;
+  // (argument errors are reported by dk_fwd below; the query returns 0 for them)
+  const size_t need = dk_fwd_workspace_bytes(&b);
+  DK_REQUIRE(need <= (size_t)DK_NOALLOC_SCRATCH_BYTES,
+             "these arguments need %zu bytes of scratch, dk_fwd_noalloc holds %zu: use dk_fwd with a workspace", need,
+             (size_t)DK_NOALLOC_SCRATCH_BYTES);
+  if (need > 0) {
+    void *ptr = nullptr;
+    if (int rc = static_scratch(&ptr)) return rc;
+    b.workspace = ptr;
+    b.workspace_bytes = (size_t)DK_NOALLOC_SCRATCH_BYTES;
+  }
+  return dk_fwd(&b);
+}
 
 size_t dk_fwd_workspace_bytes(const dk_fwd_args *a) {
   FwdParams p;

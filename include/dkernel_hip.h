@@ -109,8 +109,11 @@ typedef struct dk_lut {
   int32_t block_cols;  /* tokens per listed entry */
   int32_t group;       /* consecutive table heads known to hold identical rows (1 if unknown);
                           lets heads of a GQA group share K/V tiles inside a workgroup */
-  int32_t max_row_entries; /* largest number of entries in one row (0 if unknown); sizes the
-                              split-KV decode grid and workspace */
+  int32_t max_row_entries; /* largest number of entries in one row (0 if unknown: the number of
+                              row blocks is assumed); sizes the split-KV decode grid and
+                              workspace.  A row that holds more entries than this is still
+                              computed in full, inside the same grid and workspace: its work
+                              units only get larger shares */
   int32_t sub_block;   /* 0, or 16 / 32 with entry_width 2 and 64 x 64 tiles: the pattern's own block
                           size.  The second int of an entry is then a bit mask over the tile's
                           f x f pattern blocks, f = 64 / sub_block: bit i * f + j set = rows
@@ -163,6 +166,19 @@ int dk_fwd(const dk_fwd_args *args);
  * the split-KV kernels only with it; packed prefill runs without it too, but then every
  * workgroup scans the sequence lengths to find its own, which costs with hundreds of sequences. */
 size_t dk_fwd_workspace_bytes(const dk_fwd_args *args);
+
+/* dk_fwd for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc): the same kernels and results as dk_fwd, with
+ * the scratch (split-KV decode partials, running tile counts of packed sequences) taken from a
+ * device array that is part of the library image instead of args->workspace, which is ignored.
+ * Calls no allocating routine.  Arguments that need more than DK_NOALLOC_SCRATCH_BYTES of
+ * scratch are refused with DK_ERR_INVALID (dk_fwd_workspace_bytes tells how much a call needs).
+ * Each GPU holds one such array for the life of the process and every call on that GPU uses it:
+ * calls that overlap on one GPU (two streams, two threads) race on it -- serialise them or use
+ * dk_fwd with separate workspaces.  No counterpart in the reference, whose launchers allocate
+ * with torch on every call (dkernel/ops/sparse_attn_inference.py:67,230). */
+#define DK_NOALLOC_SCRATCH_BYTES (8u << 20)
+int dk_fwd_noalloc(const dk_fwd_args *args);
 
 /* Paged K/V cache for single-token decode (serving).  args->k / args->v point at
  * page pools: token t of sequence b lives in page block_table[b][t / page_size]

@@ -118,6 +118,15 @@ def _const_i32(device, n: int, value: int) -> Tensor:
     return t
 
 
+def _check_out(out: Optional[Tensor], q: Tensor) -> None:
+    """A caller's output tensor is written in place by the kernels: it must look like q."""
+    if out is None:
+        return
+    assert out.shape == q.shape, f"out has shape {tuple(out.shape)}, q has {tuple(q.shape)}"
+    assert out.dtype == q.dtype and out.device == q.device, "out must have q's dtype and device"
+    assert out.stride(-1) == 1, "out must have unit stride on head_dim"
+
+
 def _stream() -> C.c_void_p:
     return C.c_void_p(torch.cuda.current_stream().cuda_stream)
 
@@ -165,6 +174,7 @@ def _forward(ctx, q: Tensor, k: Tensor, v: Tensor, sm_scale: float,
         assert num_head_patterns in [num_heads, num_kv_heads]
 
     q, k, v = _unit_last(q), _unit_last(k), _unit_last(v)
+    _check_out(out, q)
     o = out if out is not None else q.new_empty(q.shape).contiguous()
     if inference is None:
         inference = (not q.requires_grad) and (not k.requires_grad) and (not v.requires_grad)
@@ -275,6 +285,7 @@ def padded_sparse_attn(q: Tensor, k: Tensor, v: Tensor, sm_scale: float,
             f'k has seqlen {k_len} while max sequence length is set to {max_seqlen}.'
     q, k, v = _unit_last(q), _unit_last(k), _unit_last(v)
     dev = q.device
+    _check_out(out, q)
     if out is None:
         # decode writes every row; padded prefill leaves the padding rows untouched, so they start at zero
         out = q.new_empty(q.shape) if q_len == 1 else q.new_zeros(q.shape)
@@ -411,6 +422,7 @@ def varlen_sparse_attn(q: Tensor, k: Tensor, v: Tensor,
     cu_q = cu_seqlens_q.to(dev, dtype=torch.int32).contiguous()
     cu_k = cu_seqlens_k.to(dev, dtype=torch.int32).contiguous()
     q, k, v = _unit_last(q), _unit_last(k), _unit_last(v)
+    _check_out(out, q)
     out = out if out is not None else q.new_empty(q.shape)
     lse = torch.full((num_heads, q.size(0)), float("-inf"), dtype=torch.float32, device=dev) if return_lse else None
 
@@ -495,7 +507,7 @@ class _sparse_attention(torch.autograd.Function):
             ctx.message = "Currently does not suppoort variable length inputs. WIP."
             res = varlen_sparse_attn(q, k, v, inf_kwargs["cu_seqlen_k"], inf_kwargs.get("cu_seqlen_q", None),
                                      sm_scale, layout_csr, max_seqlen=max_seqlen, causal=causal,
-                                     return_lse=return_lse, lut_group=lut_group, lut_max_row=lut_max_row)
+                                     out=kwargs.get("out", None), return_lse=return_lse, lut_group=lut_group, lut_max_row=lut_max_row)
             output, lse = res if return_lse else (res, None)
         else:
             assert k.size(seq_dim) <= max_seqlen, \
@@ -508,6 +520,7 @@ class _sparse_attention(torch.autograd.Function):
                 ctx.message = "Currently does not support paddings in inputs. WIP."
                 res = padded_sparse_attn(q, k, v, sm_scale, layout_csr, left_paddings=left_paddings,
                                          seqlens=seqlens, seq_dim=seq_dim, max_seqlen=max_seqlen,
+                                         out=kwargs.get("out", None),
                                          causal=causal, return_lse=return_lse, lut_group=lut_group,
                                          lut_max_row=lut_max_row)
                 output, lse = res if return_lse else (res, None)

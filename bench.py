@@ -8,8 +8,9 @@ Phi-3-small-style configuration: B=2, L=8192, 32 q heads / 8 kv heads, head_dim
 in HBM before the timed region.  Prints ONE JSON line:
 
   value     effective (sparse-counted) TFLOP/s = 4*64*64*128 * active blocks / time
-  roofline  the forward kernel against the dense bf16 MFMA peak, from HIP
-            events on the launch stream around the same timed steps
+  roofline  the forward kernel against the dense bf16 MFMA peak: median of
+            per-step HIP-event durations on the launch stream over the same
+            timed steps (extra.bwd / extra.decode carry the same object)
   cpu_baseline  the reference's dense masked-attention checker (oracle port)
             timed on this box's host cores on a bounded sample
   extra     backward (B=1, 32 MHA heads) TFLOP/s and batched-decode us/step
@@ -26,10 +27,16 @@ sys.path.insert(0, ROOT)
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16, vendor figure
 HBM_PEAK_GBS = 8000.0            # MI355X HBM3E, vendor figure
-# HBM bytes per launch of the headline forward kernel, from rocprofv3 --pmc runs of this
-# file (FETCH_SIZE x 2.00 copy calibration = 231.4 MB, WRITE_SIZE = 136.3 MB); not measured live
-FWD_TRAFFIC_BYTES = 367.7e6
+# HBM bytes per launch, from rocprofv3 --pmc runs of this file (FETCH_SIZE scaled by the copy
+# calibration + WRITE_SIZE; profiles/fwd_bwd_decode_counters.md).  Counters cannot be read from
+# inside this process, so these are quoted, not measured live; None where no counter run exists.
+TRAFFIC_BYTES = {
+    "fwd": 231.5e6 + 136.3e6,
+    "bwd": None,
+    "decode": 180.5e6 + 0.3e6,
+}
 BS, LOCAL, VERT, D = 64, 16, 8, 128
+WARM_GPU_SECONDS = 0.3           # untimed calls beyond --warmup until the clocks have settled
 
 
 def block_flops(nnz_blocks, d=D, bs=BS):
@@ -43,20 +50,48 @@ def gen(shape, g, dtype):
 
 
 def time_steps(fn, steps, warmup):
-    """(wall ms per step, HIP-event ms per step) over exactly `steps` calls."""
+    """Runs `warmup` untimed calls, keeps calling until the GPU has been busy for
+    WARM_GPU_SECONDS, then times exactly `steps` calls.  Returns (wall ms per step over the
+    whole timed region, median and mean HIP-event ms per step: one event pair per step on the
+    launch stream)."""
     import torch
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
-    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    busy = 0.0
+    while busy < WARM_GPU_SECONDS:
+        a.record()
+        for _ in range(20):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        busy += a.elapsed_time(b) * 1e-3
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    torch.cuda.synchronize()
     t0 = time.perf_counter()
-    start.record()
-    for _ in range(steps):
+    for i in range(steps):
+        marks[i].record()
         fn()
-    stop.record()
+    marks[steps].record()
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) * 1e3 / steps
-    return wall, start.elapsed_time(stop) / steps
+    per_step = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(steps))
+    median = per_step[steps // 2] if steps % 2 else 0.5 * (per_step[steps // 2 - 1] + per_step[steps // 2])
+    return wall, median, marks[0].elapsed_time(marks[steps]) / steps
+
+
+def roofline(bound, work, ms, traffic, algorithmic_bytes):
+    """work: FLOP (bound "mfma") or bytes (bound "hbm") per launch; ms: median launch duration."""
+    if bound == "mfma":
+        achieved, peak, unit = work / (ms * 1e-3) / 1e12, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s"
+    else:
+        achieved, peak, unit = work / (ms * 1e-3) / 1e9, HBM_PEAK_GBS, "GB/s"
+    return {"bound": bound, "achieved": round(achieved, 2), "peak": peak, "unit": unit,
+            "frac": round(achieved / peak, 4), "traffic": traffic,
+            "traffic_unit": "bytes per launch (rocprofv3 FETCH_SIZE / WRITE_SIZE, separate runs: "
+                            "profiles/fwd_bwd_decode_counters.md)",
+            "algorithmic_bytes": algorithmic_bytes, "kernel_ms": round(ms, 5)}
 
 
 def cpu_baseline(seconds_budget=20.0):
@@ -137,10 +172,12 @@ def main():
     k = gen((B, L, Hkv, D), g, torch.bfloat16).to(dev)
     v = gen((B, L, Hkv, D), g, torch.bfloat16).to(dev)
     with torch.no_grad():
-        wall_ms, ev_ms = time_steps(lambda: mod(q, k, v, sm, return_lse=True), args.steps, args.warmup)
+        wall_ms, ev_ms, ev_mean = time_steps(lambda: mod(q, k, v, sm, return_lse=True), args.steps, args.warmup)
     flops = block_flops(nnz) * B
     value = flops / (wall_ms * 1e-3) / 1e12
-    achieved = flops / (ev_ms * 1e-3) / 1e12
+    auto = args.impl == "auto"
+    # q + k + v read once, o + lse written once
+    fwd_bytes = (2 * B * L * Hq * D + 2 * B * L * Hkv * D) * 2 + B * L * Hq * 4
 
     out = {
         "metric": "effective fwd TFLOP/s, causal block-sparse prefill, L=8192 d=128 bf16, 1 MI355X",
@@ -151,12 +188,9 @@ def main():
         "config": {"workload": "prefill fwd + LSE: B=2 L=8192 Hq=32 Hkv=8 d=128 bf16, block 64, "
                                "local 16, vert 8, heterogeneous heads, causal",
                    "active_blocks_per_batch": nnz, "flop_per_step": flops, "impl": args.impl},
-        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_BF16_PEAK_TFLOPS,
-                     "unit": "TFLOP/s", "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4),
-                     "traffic": FWD_TRAFFIC_BYTES if args.impl == "auto" else None,
-                     "traffic_unit": "bytes per launch (rocprofv3 counters, separate run)",
-                     "algorithmic_bytes": 201.3e6 + 136.3e6, "kernel_ms": round(ev_ms, 4)},
+        "roofline": roofline("mfma", flops, ev_ms, TRAFFIC_BYTES["fwd"] if auto else None, fwd_bytes),
     }
+    out["roofline"]["kernel_ms_mean"] = round(ev_mean, 5)
     del q, k, v
 
     if not args.no_extra:
@@ -171,13 +205,18 @@ def main():
         def bwd():
             torch.autograd.grad(o2, (q2, k2, v2), do2, retain_graph=True)
         steps2 = max(5, args.steps // 4)
-        w2, e2 = time_steps(bwd, steps2, max(2, args.warmup // 4))
+        w2, e2, _ = time_steps(bwd, steps2, max(2, args.warmup // 4))
         with torch.no_grad():
-            wf, ef = time_steps(lambda: mod2(q2, k2, v2, sm), steps2, 2)
-        extra["bwd"] = {"workload": "dQ,dK,dV: B=1 L=8192 H=32 (MHA) d=128 bf16, same pattern",
-                        "tflops": round(2.5 * block_flops(nnz2) / (e2 * 1e-3) / 1e12, 2),
+            wf, ef, _ = time_steps(lambda: mod2(q2, k2, v2, sm), steps2, 2)
+        bwd_flops = 2.5 * block_flops(nnz2)
+        # q, k, v, o, dO read and dq, dk, dv written once (bf16), lse read (fp32)
+        bwd_bytes = 8 * L * 32 * D * 2 + L * 32 * 4
+        extra["bwd"] = {"workload": "dQ,dK,dV: B=1 L=8192 H=32 (MHA) d=128 bf16, same pattern "
+                                    "(dQ pass + dK/dV pass, 5 of the 7 executed GEMMs counted)",
+                        "tflops": round(bwd_flops / (e2 * 1e-3) / 1e12, 2),
                         "ms": round(e2, 4), "frac_of_mfma_peak":
-                        round(2.5 * block_flops(nnz2) / (e2 * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+                        round(bwd_flops / (e2 * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+                        "roofline": roofline("mfma", bwd_flops, e2, TRAFFIC_BYTES["bwd"] if auto else None, bwd_bytes),
                         "fwd_mha_tflops": round(block_flops(nnz2) / (ef * 1e-3) / 1e12, 2)}
         del q2, k2, v2, do2, o2
         # ---- C3: batched decode over left-padded KV --------------------------
@@ -209,13 +248,14 @@ def main():
                 kd, vd = kv_sets[step[0] & 1]
                 step[0] += 1
                 return mod(qd, kd, vd, sm, left_paddings=left)
-            wd, ed = time_steps(decode_step, args.steps, args.warmup)
+            wd, ed, _ = time_steps(decode_step, args.steps, args.warmup)
         extra["decode"] = {"workload": "32 seqs x 1 token, Hq=32 Hkv=8 d=128 bf16, KV len U[1024,8192] left-padded, "
                                        "2 K/V sets alternated (working set > Infinity Cache)",
                            "us_per_step": round(wd * 1e3, 2), "kernel_us": round(ed * 1e3, 2),
                            "algorithmic_MB": round(byts / 1e6, 2),
                            "achieved_GBs": round(byts / (ed * 1e-3) / 1e9, 1),
-                           "frac_of_hbm_peak": round(byts / (ed * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+                           "frac_of_hbm_peak": round(byts / (ed * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                           "roofline": roofline("hbm", byts, ed, TRAFFIC_BYTES["decode"] if auto else None, byts)}
         out["extra"] = extra
 
     if not args.no_cpu:

@@ -26,7 +26,7 @@ using dk::fail;
 
 extern "C" {
 
-int dk_version(void) { return 200; /* 0.2.0 */ }
+int dk_version(void) { return 300; /* 0.3.0 */ }
 const char *dk_last_error(void) { return dk::g_err; }
 
 // dkernel/utils.py:157-215.  Head h of the pattern belongs to kv head

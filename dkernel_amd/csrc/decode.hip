@@ -155,11 +155,18 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(2, 2))) 
   using KV = typename std::conditional<KV8, uint8_t, T>::type;  // element type of the K/V memory
   const KV *kbase = (const KV *)p.k.ptr + kvh * p.k.sh + (PAGED ? 0 : sq.b * p.k.sb + (int64_t)sq.k_start * p.k.st);
   const KV *vbase = (const KV *)p.v.ptr + kvh * p.v.sh + (PAGED ? 0 : sq.b * p.v.sb + (int64_t)sq.k_start * p.v.st);
+  // K/V bytes are read once per step: non-temporal loads keep them from displacing each other in
+  // the memory-side cache (measured 44.6 -> 40.5 us per step on 32 sequences of 1K-8K tokens)
   auto load8 = [](const KV *src) -> uint4 {  // 8 head dims starting at src, as T
-    if constexpr (KV8)
-      return fp8x8_to<T>(*reinterpret_cast<const uint2 *>(src));
-    else
-      return *reinterpret_cast<const uint4 *>(src);
+    if constexpr (KV8) {
+      typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+      const u32x2 w = __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(src));
+      return fp8x8_to<T>(make_uint2(w[0], w[1]));
+    } else {
+      typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+      const u32x4 w = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src));
+      return make_uint4(w[0], w[1], w[2], w[3]);
+    }
   };
 
   // PAGED: page numbers of the whole unit in one vector load, four lanes per table entry (a

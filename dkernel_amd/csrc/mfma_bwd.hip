@@ -291,40 +291,42 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, D == 64 
 // ---------------------------------------------------------------------------
 // dK / dV pass
 // ---------------------------------------------------------------------------
-// One workgroup = one 64-key column block of one kv head, 8 waves.  The four
-// 32 x 32 (q rows x keys) quadrants of a block are each worked on by a pair of
-// waves that sit on the same SIMD:
+// One workgroup = one 64-key column block of one kv head, 4 waves, two workgroups per CU (the
+// start-up and close-down of one column then overlap with the other workgroup's loop, and the
+// two workgroups' barriers are independent).  A listed q block is worked on in two steps of 32
+// q rows; in each step the two 32 x 32 (q rows x keys) quadrants are each shared by a pair of
+// waves:
 //   the S wave:   S = Q K^T, P = exp(S - lse), dV^T += dO^T P     (K fragments and dV in registers)
 //   the dP wave:  dP = dO V^T, dS = P (dP - delta), dK^T += Q^T dS (V fragments and dK in registers)
-// so that each wave holds half of the accumulators and fits in the 256
-// registers of two waves per SIMD.  P goes from the S wave to the dP wave
-// through LDS in fp32, exactly as computed.  The dP wave finishes a block one
-// iteration late (after the next block's barrier has published P), so one
-// barrier per block is enough: Q tiles and the lse / delta vectors live one
-// iteration longer than dO tiles (rings of 4 and 3 stages), and tile loads run
-// two blocks ahead.
+// so that each wave holds the accumulators of one matrix for 32 keys and fits in the 256
+// registers of two waves per SIMD.  P goes from the S wave to the dP wave through LDS in fp32,
+// exactly as computed.  The dP wave finishes a step one iteration late (after the next step's
+// barrier has published P), so one barrier per step is enough: Q tiles and the lse / delta
+// vectors live one iteration longer than dO tiles (rings of 4 and 3 stages of 32-row tiles), and
+// tile loads run two steps ahead.
 template <int D>
 struct DkdvSmem {
   using TL = Tile<D>;
+  static constexpr int kRows = 32;                            // q rows per step
+  static constexpr int kTile = kRows * TL::kRowBytes;         // one 32-row tile
   static constexpr int kQStages = 4, kDoStages = 3, kAhead = 2;
   static constexpr int kQ = 0;                                // Q ring
-  static constexpr int kDo = kQ + kQStages * TL::kBytes;      // dO ring
-  static constexpr int kVec = kDo + kDoStages * TL::kBytes;   // per Q stage: lse[64], delta[64]
-  static constexpr int kX = kVec + kQStages * 512;            // P exchange: [pair 4][buffer 2][16][64] floats
-  static constexpr int kLoop = kX + 4 * 2 * 4096;
-  static constexpr int kRed = 2 * 2 * (D / 32) * 16 * 64 * 4;  // epilogue: [role][nh][DT*16][64] floats
-  static constexpr int kBytes = kLoop > kRed ? kLoop : kRed;
+  static constexpr int kDo = kQ + kQStages * kTile;           // dO ring
+  static constexpr int kVec = kDo + kDoStages * kTile;        // per Q stage: lse[32], delta[32]
+  static constexpr int kX = kVec + kQStages * 256;            // P exchange: [pair 2][buffer 2][16][64] floats
+  static constexpr int kBytes = kX + 2 * 2 * 4096;
 };
 
 template <typename T, int D, bool PAD, bool SUB>
-__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void mfma_dkdv_kernel(const BwdParams p, int head_split) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void mfma_dkdv_kernel(const BwdParams p, int head_split) {
   using M = Mma<T>;
   using vec8 = typename M::vec8;
   using TL = Tile<D>;
   using S = DkdvSmem<D>;
-  constexpr int NT = 512;
+  constexpr int NT = 256;
   constexpr int KS = D / 16, DT = D / 32;
-  constexpr int LPT = 2 * TileLoader<D, NT>::kChunks + 1;  // load instructions per wave per block
+  using Loader = TileLoader<D, NT, PAD, S::kRows>;
+  constexpr int LPT = 2 * Loader::kChunks + 1;  // load instructions per wave per step
   // SUB: table entries are (row block, bit mask over the pattern blocks inside the 64 x 64 tile)
   constexpr int EW = SUB ? 2 : 1;  // ints per table entry
   extern __shared__ __align__(16) char smem[];
@@ -341,8 +343,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int gq_end = head_split ? gq_first + 1 : ratio;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int pair = wave & 3, nh = wave & 1, mh = (wave >> 1) & 1;
-  const bool dp_wave = wave >= 4;
+  const int nh = wave & 1;  // key half; also the index of the (S wave, dP wave) pair
+  const bool dp_wave = wave >= 2;
   const int n = lane & 31, g = lane >> 5;
   const int key = cb * 64 + nh * 32 + n;
   const bool key_ok = key < sq.k_len;
@@ -358,14 +360,20 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       if (key_ok && (!PAD || ks * 16 + g * 8 < p.D)) a = *reinterpret_cast<const uint4 *>(src + ks * 16 + g * 8);
       kvf[ks] = as_vec8<vec8>(a);
     }
+    // The fragments pass through an empty asm statement: the compiler then waits for their
+    // loads here, once.  Left to itself it waits at their first use inside the loop, in every
+    // iteration, with vmcnt(0) -- which also waits for the tile copies in flight (issued from
+    // inline assembly, so unknown to its counter bookkeeping) and undoes the prefetch.
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(kvf[ks]));
   }
-  floatx16 acc[DT];  // dV^T (S wave) or dK^T (dP wave): d x keys
+  floatx16 acc[DT];  // dV^T (S wave) or dK^T (dP wave): d x keys, summed over every q row of the column
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[dt][r] = 0.f;
 
-  TileLoader<D, NT, PAD> qload, doload;
+  Loader qload, doload;
   qload.init(tid, p.q.st, p.D);
   doload.init(tid, p.dout.st, p.D);
   if constexpr (PAD) {  // the slots of the head dims beyond p.D stay zero in every Q / dO stage
@@ -374,9 +382,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   }
   int rd[KS], tr[DT][2];
 #pragma unroll
-  for (int ks = 0; ks < KS; ++ks) rd[ks] = TL::off(mh * 32 + n, 2 * ks + g);
+  for (int ks = 0; ks < KS; ++ks) rd[ks] = TL::off(n, 2 * ks + g);
   transposed_offsets<D>(lane, tr);
-  float *xbuf = reinterpret_cast<float *>(smem + S::kX) + pair * 2 * 1024;  // this pair's two P buffers
+  float *xbuf = reinterpret_cast<float *>(smem + S::kX) + nh * 2 * 1024;  // this pair's two P buffers
 
   for (int gq = gq_first; gq < gq_end; ++gq) {
     const int h = kvh * ratio + gq;
@@ -384,54 +392,52 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     int e0 = 0, e1 = 0;
     if (cb < p.csc.num_rows)
       scalar_load2(p.csc.ptr + lh * p.csc.ptr_sh + cb, p.csc.ptr + lh * p.csc.ptr_sh + cb + 1, e0, e1);
-    const int nblk = e1 - e0;
+    const int nstep = 2 * (e1 - e0);  // two steps of 32 q rows per listed block
     const int32_t *rows = p.csc.idx + lh * p.csc.idx_sh + e0 * EW;
     const T *qbase = (const T *)p.q.ptr + sq.b * p.q.sb + h * p.q.sh;
     const T *dobase = (const T *)p.dout.ptr + sq.b * p.dout.sb + h * p.dout.sh;
     const float *lsebase = p.lse.ptr + sq.b * p.lse.sb + h * p.lse.sh;
     const float *deltabase = p.delta + ((int64_t)sq.b * p.Hq + h) * p.seqs.max_q_len;
 
-    // asynchronous copy of q block rows[t]: Q and dO tiles and the 64 lse / 64 delta values of
-    // its rows (even waves copy lse, odd waves delta; they all write the same values, so that
-    // every wave issues the same number of load instructions).  Returns false when rows had
-    // to be zero-filled, i.e. when the per-wave load count is not LPT.
-    auto issue = [&](int rbq, int qstage, int dostage) -> bool {
-      const int qi0 = rbq * 64 - sq.past;  // query index of the tile's first row
+    // asynchronous copy of half `half` of q block rbq: Q and dO tiles and the 32 lse / 32 delta
+    // values of its rows (lanes 0..31 copy lse, lanes 32..63 delta; every wave copies the same
+    // values, so that every wave issues the same number of load instructions).  Returns false
+    // when rows had to be zero-filled, i.e. when the per-wave load count is not LPT.
+    auto issue = [&](int rbq, int half, int qstage, int dostage) -> bool {
+      const int qi0 = rbq * 64 + half * 32 - sq.past;  // query index of the tile's first row
       // rows before the first query (qi < 0, when k is longer than q) and beyond the last are zero-filled
-      const int lo = rbq < 0 ? 64 : -qi0, hi = sq.q_len - qi0;
+      const int lo = rbq < 0 ? S::kRows : -qi0, hi = sq.q_len - qi0;
       const bool full = qload.issue(reinterpret_cast<const char *>(qbase + (int64_t)qi0 * p.q.st), lo, hi,
-                                    smem + S::kQ + qstage * TL::kBytes);
+                                    smem + S::kQ + qstage * S::kTile);
       doload.issue(reinterpret_cast<const char *>(dobase + (int64_t)qi0 * p.dout.st), lo, hi,
-                   smem + S::kDo + dostage * TL::kBytes);
-      const int row = lane;
-      const bool is_delta = (wave & 1) != 0;
-      char *dst = smem + S::kVec + qstage * 512 + (is_delta ? 256 : 0);
+                   smem + S::kDo + dostage * S::kTile);
+      const int row = lane & 31;
+      const bool is_delta = lane >= 32;
+      char *dst = smem + S::kVec + qstage * 256;
       if (full) {
-        // wave-uniform base (row qi0) + this lane's row
-        const float *src0 = is_delta ? deltabase + qi0 : lsebase + (int64_t)qi0 * p.lse.st;
-        const uint32_t voff = (uint32_t)(row * (is_delta ? 1 : (int)p.lse.st)) * 4u;
-        lds_dma4(reinterpret_cast<const char *>(src0), voff, lds_address(dst));
-      } else if (wave < 2) {
+        const float *src = is_delta ? deltabase + qi0 + row : lsebase + (int64_t)(qi0 + row) * p.lse.st;
+        lds_dma4_lane(src, lds_address(dst));
+      } else if (wave == 0) {
         // rows outside the sequence: lse = +inf makes their probabilities 0
         const int qi = qi0 + row;
         float x = is_delta ? 0.f : INFINITY;
         if (row >= lo && row < hi) x = is_delta ? deltabase[qi] : lsebase[(int64_t)qi * p.lse.st];
-        reinterpret_cast<float *>(dst)[row] = x;
+        reinterpret_cast<float *>(dst)[lane] = x;
       }
       return full;
     };
 
-    // second half of the dP wave's work on block u (whose P the S wave published before the
+    // second half of the dP wave's work on step u (whose P the S wave published before the
     // last barrier): dS = P (dP - delta), dK^T += Q^T dS
     auto finish_dk = [&](int u, int qstage, const floatx16 &dp) {
-      const char *qs_ = smem + S::kQ + qstage * TL::kBytes;
-      const float *delta_s = reinterpret_cast<const float *>(smem + S::kVec + qstage * 512) + 64;
+      const char *qs_ = smem + S::kQ + qstage * S::kTile;
+      const float *delta_s = reinterpret_cast<const float *>(smem + S::kVec + qstage * 256) + 32;
       const float *x = xbuf + (u & 1) * 1024;
       float ds[16];
 #pragma unroll
       for (int r4 = 0; r4 < 4; ++r4) {
         const float4 p4 = *reinterpret_cast<const float4 *>(x + (r4 * 64 + lane) * 4);
-        const float4 d4 = *reinterpret_cast<const float4 *>(delta_s + mh * 32 + r4 * 8 + g * 4);
+        const float4 d4 = *reinterpret_cast<const float4 *>(delta_s + r4 * 8 + g * 4);
         ds[r4 * 4 + 0] = p4.x * (dp[r4 * 4 + 0] - d4.x);  // without sm_scale
         ds[r4 * 4 + 1] = p4.y * (dp[r4 * 4 + 1] - d4.y);
         ds[r4 * 4 + 2] = p4.z * (dp[r4 * 4 + 2] - d4.z);
@@ -440,7 +446,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
       for (int t2 = 0; t2 < 2; ++t2) {
         const vec8 dsb = M::pack(ds + t2 * 8);
-        const int rowoff = (mh * 32 + t2 * 16) * TL::kRowBytes;
+        const int rowoff = t2 * 16 * TL::kRowBytes;
         vec8 qt[DT];
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) qt[dt] = lds_read_tr8<vec8>(qs_ + rowoff + tr[dt][0], qs_ + rowoff + tr[dt][1]);
@@ -453,38 +459,42 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // are not merged through a join every iteration.
     auto run_head = [&](auto role_tag) {
     constexpr bool kDp = decltype(role_tag)::value;
-    int issued = 0, iq = 0, ido = 0;  // next block to request and its ring positions
-    bool exact = true;                // every wave has issued exactly LPT load instructions per outstanding block
-    static_assert(S::kAhead == 2, "the first two table entries are read together");
-    if (nblk > 0) {
-      int r0, r1;
-      scalar_load2(rows, rows + (nblk > 1 ? EW : 0), r0, r1);  // one round trip for both
-      for (int i = 0; i < S::kAhead && issued < nblk; ++i, ++issued) {
-        exact = issue(i == 0 ? r0 : r1, iq, ido) && exact;
+    int issued = 0, iq = 0, ido = 0;  // next step to request and its ring positions
+    bool exact = true;                // every wave has issued exactly LPT load instructions per outstanding step
+    static_assert(S::kAhead == 2, "the first block's two steps are requested together");
+    int rb_next = 0;                  // q block of the next step to request (steps 2k and 2k + 1 share block k)
+    if (nstep > 0) {
+      rb_next = scalar_load(rows);
+      for (int i = 0; i < S::kAhead; ++i, ++issued) {
+        exact = issue(rb_next, i, iq, ido) && exact;
         iq = iq + 1 == S::kQStages ? 0 : iq + 1;
         ido = ido + 1 == S::kDoStages ? 0 : ido + 1;
       }
     }
     floatx16 dp_prev;
-    int cq = 0, cdo = 0, pq = 0;  // ring positions of block t (Q, dO) and of block t - 1 (Q)
-    for (int t = 0; t < nblk; ++t) {
+    int cq = 0, cdo = 0, pq = 0;  // ring positions of step t (Q, dO) and of step t - 1 (Q)
+    int rbq = 0, bits = 0;        // S wave: q block (and its mask) of the current step
+    for (int t = 0; t < nstep; ++t) {
+      const int half = t & 1;
       wait_tiles_ahead<LPT>(exact ? issued - t - 1 : 0);
-      __syncthreads();  // block t is visible, so is P of block t - 1; the stages of block t - 2 are free
-      if (issued < nblk) {
-        exact = issue(scalar_load(rows + issued * EW), iq, ido) && exact;
+      __syncthreads();  // step t is visible, so is P of step t - 1; the stages of step t - 2 are free
+      if (issued < nstep) {
+        if ((issued & 1) == 0) rb_next = scalar_load(rows + (issued >> 1) * EW);
+        exact = issue(rb_next, issued & 1, iq, ido) && exact;
         iq = iq + 1 == S::kQStages ? 0 : iq + 1;
         ido = ido + 1 == S::kDoStages ? 0 : ido + 1;
         ++issued;
       }
-      const char *qs_ = smem + S::kQ + cq * TL::kBytes, *dos_ = smem + S::kDo + cdo * TL::kBytes;
+      const char *qs_ = smem + S::kQ + cq * S::kTile, *dos_ = smem + S::kDo + cdo * S::kTile;
       if constexpr (!kDp) {
-        int rbq, bits = 0;
-        if constexpr (SUB)
-          scalar_load2(rows + t * EW, rows + t * EW + 1, rbq, bits);
-        else
-          rbq = scalar_load(rows + t);
-        const int pos0 = rbq * 64 + mh * 32;  // first q position of this wave's half
-        const float *lse_s = reinterpret_cast<const float *>(smem + S::kVec + cq * 512);
+        if (half == 0) {
+          if constexpr (SUB)
+            scalar_load2(rows + (t >> 1) * EW, rows + (t >> 1) * EW + 1, rbq, bits);
+          else
+            rbq = scalar_load(rows + (t >> 1));
+        }
+        const int pos0 = rbq * 64 + half * 32;  // first q position of this step
+        const float *lse_s = reinterpret_cast<const float *>(smem + S::kVec + cq * 256);
         // S = Q K^T : rows = 32 q positions, cols = 32 keys
         floatx16 sc;
 #pragma unroll
@@ -498,15 +508,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         }
         // first dO^T operands do not depend on P
         vec8 dot[DT];
-        {
-          const int rowoff = (mh * 32) * TL::kRowBytes;
 #pragma unroll
-          for (int dt = 0; dt < DT; ++dt) dot[dt] = lds_read_tr8<vec8>(dos_ + rowoff + tr[dt][0], dos_ + rowoff + tr[dt][1]);
-        }
+        for (int dt = 0; dt < DT; ++dt) dot[dt] = lds_read_tr8<vec8>(dos_ + tr[dt][0], dos_ + tr[dt][1]);
         // P = exp2(S scale - lse log2e).  Rows outside the sequence arrive with lse = +inf
         // (P = 0).  A row that saw no key has lse = -inf, but then every one of its entries
         // here is masked by causality and the select below discards the infinite value, so no
-        // conversion is needed.  Masks are applied only in blocks that need them (the diagonal
+        // conversion is needed.  Masks are applied only in steps that need them (the diagonal
         // block and the last, partial column block): wave-uniform choice between two loops.
         const bool edge = (p.causal && (cb * 64 + nh * 32 + 31 > pos0)) || cb * 64 + 63 >= sq.k_len;
         // last visible q-row offset test: key is visible to row pos iff key <= pos
@@ -514,8 +521,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         float *x = xbuf + (t & 1) * 1024;
 #pragma unroll
         for (int r4 = 0; r4 < 4; ++r4) {
-          // registers 4*r4 .. +3 are q rows mh*32 + 8*r4 + 4g + {0..3}
-          const float4 l4 = *reinterpret_cast<const float4 *>(lse_s + mh * 32 + r4 * 8 + g * 4);
+          // registers 4*r4 .. +3 are q rows 8*r4 + 4g + {0..3} of the step
+          const float4 l4 = *reinterpret_cast<const float4 *>(lse_s + r4 * 8 + g * 4);
           const float lr[4] = {l4.x, l4.y, l4.z, l4.w};
 #pragma unroll
           for (int i = 0; i < 4; ++i)
@@ -527,14 +534,14 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         }
         if constexpr (SUB) {
           // pattern blocks of the tile that are not attended: bit (row part) * f + (key part); this
-          // lane's key is nh 32 + n, register r is q row mh 32 + 8 (r / 4) + 4 g + r % 4
+          // lane's key is nh 32 + n, register r is q row half 32 + 8 (r / 4) + 4 g + r % 4
           const int lb = p.csc.sub_block == 16 ? 4 : 5, f = 64 >> lb;
           const int full = f == 4 ? 0xffff : 0xf;
           if ((bits & full) != full) {  // wave-uniform
             const int key_bits = bits >> ((nh * 32 + n) >> lb);
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-              const int row_part = (mh * 32 + (r >> 2) * 8) >> lb;
+              const int row_part = (half * 32 + (r >> 2) * 8) >> lb;
               sc[r] = ((key_bits >> (row_part * f)) & 1) ? sc[r] : 0.f;
             }
           }
@@ -554,13 +561,13 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           for (int dt = 0; dt < DT; ++dt) {
             acc[dt] = M::mma(dot[dt], pb, acc[dt]);
             if (t2 == 0) {
-              const int rowoff = (mh * 32 + 16) * TL::kRowBytes;
+              const int rowoff = 16 * TL::kRowBytes;
               dot[dt] = lds_read_tr8<vec8>(dos_ + rowoff + tr[dt][0], dos_ + rowoff + tr[dt][1]);
             }
           }
         }
       } else {
-        // second half of block t - 1 first: it frees dp_prev for this block's dP
+        // second half of step t - 1 first: it frees dp_prev for this step's dP
         if (t > 0) finish_dk(t - 1, pq, dp_prev);
         // dP = dO V^T
 #pragma unroll
@@ -577,28 +584,20 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       cq = cq + 1 == S::kQStages ? 0 : cq + 1;
       cdo = cdo + 1 == S::kDoStages ? 0 : cdo + 1;
     }
-    __syncthreads();  // P of the last block is visible
+    __syncthreads();  // P of the last step is visible
     if constexpr (kDp) {
-      if (nblk > 0) finish_dk(nblk - 1, pq, dp_prev);
+      if (nstep > 0) finish_dk(nstep - 1, pq, dp_prev);
     }
     };
     if (dp_wave)
       run_head(BoolConst<true>{});
     else
       run_head(BoolConst<false>{});
-    __syncthreads();  // every wave is done with every stage before the next head reuses them
+    if (gq + 1 < gq_end) __syncthreads();  // every wave is done with every stage before the next head reuses them
   }
 
-  // sum the two q-row halves: waves with mh = 1 hand their partials to mh = 0
-  float *red = reinterpret_cast<float *>(smem) + ((dp_wave ? 2 : 0) + nh) * DT * 16 * 64;
-  if (mh == 1) {
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) red[(dt * 16 + r) * 64 + lane] = acc[dt][r];
-  }
-  __syncthreads();
-  if (mh == 1 || !key_ok) return;
+  // every wave holds the finished dV^T (S wave) or dK^T (dP wave) of its 32 keys
+  if (!key_ok) return;
   const float out_scale = dp_wave ? p.sm_scale : 1.f;
   const TensorView &outv = dp_wave ? p.dk : p.dv;
   const int64_t out_off = sq.b * outv.sb + out_head * outv.sh + (int64_t)key * outv.st;
@@ -609,10 +608,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
       for (int r4 = 0; r4 < 4; ++r4) {
         float4 o4;
-        o4.x = (acc[dt][r4 * 4 + 0] + red[(dt * 16 + r4 * 4 + 0) * 64 + lane]) * out_scale;
-        o4.y = (acc[dt][r4 * 4 + 1] + red[(dt * 16 + r4 * 4 + 1) * 64 + lane]) * out_scale;
-        o4.z = (acc[dt][r4 * 4 + 2] + red[(dt * 16 + r4 * 4 + 2) * 64 + lane]) * out_scale;
-        o4.w = (acc[dt][r4 * 4 + 3] + red[(dt * 16 + r4 * 4 + 3) * 64 + lane]) * out_scale;
+        o4.x = acc[dt][r4 * 4 + 0] * out_scale;
+        o4.y = acc[dt][r4 * 4 + 1] * out_scale;
+        o4.z = acc[dt][r4 * 4 + 2] * out_scale;
+        o4.w = acc[dt][r4 * 4 + 3] * out_scale;
         if (!PAD || dt * 32 + r4 * 8 + g * 4 < p.D) *reinterpret_cast<float4 *>(outp + dt * 32 + r4 * 8 + g * 4) = o4;
       }
     return;
@@ -624,10 +623,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     for (int r4 = 0; r4 < 4; ++r4) {
       T o4[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int r = r4 * 4 + i;
-        o4[i] = from_float<T>((acc[dt][r] + red[(dt * 16 + r) * 64 + lane]) * out_scale);
-      }
+      for (int i = 0; i < 4; ++i) o4[i] = from_float<T>(acc[dt][r4 * 4 + i] * out_scale);
       if (!PAD || dt * 32 + r4 * 8 + g * 4 < p.D)
         *reinterpret_cast<uint2 *>(outp + dt * 32 + r4 * 8 + g * 4) = *reinterpret_cast<const uint2 *>(o4);
     }
@@ -744,7 +740,7 @@ static int launch_bwd_td(const BwdParams &p, void *workspace, size_t workspace_b
     float *part_k = (float *)workspace, *part_v = part_k + (int64_t)s.batch * p.Hq * keys * p.D;
     pp.dk = TensorView{part_k, p.Hq * keys * p.D, keys * p.D, p.D};
     pp.dv = TensorView{part_v, p.Hq * keys * p.D, keys * p.D, p.D};
-    hipLaunchKernelGGL((mfma_dkdv_kernel<T, D, PAD, SUB>), dim3(p.Hq, cblocks, s.batch), dim3(512), smem_dkdv, stream, pp, 1);
+    hipLaunchKernelGGL((mfma_dkdv_kernel<T, D, PAD, SUB>), dim3(p.Hq, cblocks, s.batch), dim3(256), smem_dkdv, stream, pp, 1);
     DK_HIP_CHECK(hipGetLastError());
     const int64_t total = (int64_t)s.batch * p.Hkv * keys * (p.D / 8);
     hipLaunchKernelGGL((dkdv_group_sum_kernel<T>), dim3((unsigned)cdiv64(total, 256), 2), dim3(256), 0, stream, part_k,
@@ -752,7 +748,7 @@ static int launch_bwd_td(const BwdParams &p, void *workspace, size_t workspace_b
     DK_HIP_CHECK(hipGetLastError());
     return DK_OK;
   }
-  hipLaunchKernelGGL((mfma_dkdv_kernel<T, D, PAD, SUB>), dim3(p.Hkv, cblocks, s.batch), dim3(512), smem_dkdv, stream, p, 0);
+  hipLaunchKernelGGL((mfma_dkdv_kernel<T, D, PAD, SUB>), dim3(p.Hkv, cblocks, s.batch), dim3(256), smem_dkdv, stream, p, 0);
   DK_HIP_CHECK(hipGetLastError());
   return DK_OK;
 }

@@ -198,6 +198,13 @@ __device__ __forceinline__ void lds_dma4(const char *gbase, uint32_t voff, uint3
                : "v"(voff), "s"(uniform_address(gbase)), "s"(__builtin_amdgcn_readfirstlane(lds_base))
                : "memory");
 }
+// The same with a full address per lane (lanes of one copy may read different arrays).
+__device__ __forceinline__ void lds_dma4_lane(const void *lane_ptr, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off"
+               :
+               : "v"(lane_ptr), "s"(__builtin_amdgcn_readfirstlane(lds_base))
+               : "memory");
+}
 
 // Asynchronous global -> LDS copy of one tile by NT threads, straight into LDS
 // (LDS DMA: no staging registers, no ds_write): a wave instruction moves 64 x 16 bytes
@@ -213,10 +220,13 @@ __device__ __forceinline__ void lds_dma4(const char *gbase, uint32_t voff, uint3
 // tile area that was zeroed once (zero_tiles) keeps zeros there for good.
 // Every row has chunks inside the real width, so every wave still issues
 // exactly kChunks load instructions per tile.
-template <int D, int NT, bool PAD = false>
+//
+// ROWS: rows of the tile (64, or 32 for half tiles; the swizzle only depends on row & 15).
+template <int D, int NT, bool PAD = false, int ROWS = 64>
 struct TileLoader {
   static constexpr int kCPR = D / 8;
-  static constexpr int kChunks = 64 * kCPR / NT;
+  static constexpr int kChunks = ROWS * kCPR / NT;
+  static_assert(kChunks >= 1 && ROWS * kCPR % NT == 0, "every thread copies the same number of chunks");
   uint32_t goff[kChunks];  // global byte offset of this thread's chunk c inside the 64-row block
   int row0;                // first row this thread's wave covers with chunk 0 (wave-uniform)
   int lane_row, lane_byte;
@@ -243,7 +253,7 @@ struct TileLoader {
   // gblk (first byte of the 64-row block) is wave-uniform.
   __device__ __forceinline__ bool issue(const char *gblk, int lo, int hi, char *tile) const {
     const uint32_t base = lds_address(tile) + row0 * Tile<D>::kRowBytes;
-    if (lo <= 0 && hi >= 64) {
+    if (lo <= 0 && hi >= ROWS) {
 #pragma unroll
       for (int c = 0; c < kChunks; ++c)
         if (!PAD || ((inside >> c) & 1)) lds_dma16(gblk, goff[c], base + c * (NT / kCPR) * Tile<D>::kRowBytes);

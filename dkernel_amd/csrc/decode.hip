@@ -506,7 +506,7 @@ bool decode_supported(const FwdParams &p, int dtype) {
   const int ratio = p.Hq / p.Hkv;
   const bool shared_row = p.csr.num_heads == 1 || (p.csr.num_heads == p.Hkv && p.Hkv != p.Hq) || ratio == 1 ||
                           (p.csr.num_heads == p.Hq && p.csr.group % ratio == 0);
-  return (dtype == DK_BF16 || dtype == DK_F16) && mfma_head_dim_ok(p.D) && p.csr.block_rows == 64 &&
+  return (dtype == DK_BF16 || dtype == DK_F16) && mfma_head_dim_ok(p.D) && p.D <= 128 && p.csr.block_rows == 64 &&
          p.csr.block_cols == 64 && p.vec_ok &&
          (p.csr.entry_width == 1 || p.csr.sub_block != 0) &&
          (p.seqs.packed ? (p.seqs.packed & 2) != 0 : p.seqs.max_q_len == 1) && ratio <= 32 && shared_row && p.causal;

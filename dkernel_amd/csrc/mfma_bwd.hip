@@ -44,7 +44,7 @@ struct BoolConst {
 // dQ pass
 // ---------------------------------------------------------------------------
 template <typename T, int D, bool PAD, bool SUB>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, D == 64 ? 3 : 2))) void mfma_dq_kernel(const BwdParams p,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 1 : 2, D == 64 ? 3 : D == 256 ? 1 : 2))) void mfma_dq_kernel(const BwdParams p,
                                                                                                    int tiles_y) {
   using M = Mma<T>;
   using vec8 = typename M::vec8;
@@ -318,7 +318,7 @@ struct DkdvSmem {
 };
 
 template <typename T, int D, bool PAD, bool SUB>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void mfma_dkdv_kernel(const BwdParams p, int head_split) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 1 : 2, D == 256 ? 1 : 2))) void mfma_dkdv_kernel(const BwdParams p, int head_split) {
   using M = Mma<T>;
   using vec8 = typename M::vec8;
   using TL = Tile<D>;
@@ -631,6 +631,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
 // Explicit instantiations: with only the implicit ones the fp16 host stubs of
 // these kernels are not emitted by this compiler version.
+// (256-wide tiles: the zero-padding instantiations only; they also take head_dim 256 itself)
+template __global__ void mfma_dq_kernel<bf16_t, 256, true, false>(const BwdParams, int);
+template __global__ void mfma_dq_kernel<bf16_t, 256, true, true>(const BwdParams, int);
+template __global__ void mfma_dq_kernel<f16_t, 256, true, false>(const BwdParams, int);
+template __global__ void mfma_dq_kernel<f16_t, 256, true, true>(const BwdParams, int);
+template __global__ void mfma_dkdv_kernel<bf16_t, 256, true, false>(const BwdParams, int);
+template __global__ void mfma_dkdv_kernel<bf16_t, 256, true, true>(const BwdParams, int);
+template __global__ void mfma_dkdv_kernel<f16_t, 256, true, false>(const BwdParams, int);
+template __global__ void mfma_dkdv_kernel<f16_t, 256, true, true>(const BwdParams, int);
 template __global__ void mfma_dq_kernel<bf16_t, 128, false, false>(const BwdParams, int);
 template __global__ void mfma_dq_kernel<bf16_t, 128, true, false>(const BwdParams, int);
 template __global__ void mfma_dq_kernel<bf16_t, 128, false, true>(const BwdParams, int);
@@ -756,6 +765,9 @@ static int launch_bwd_td(const BwdParams &p, void *workspace, size_t workspace_b
 // head dims below the tile width (64 or 128) run the zero-padded instantiation
 template <typename T>
 static int launch_bwd_t(const BwdParams &p, void *ws, size_t ws_bytes, hipStream_t stream) {
+  if (p.D > 128)  // 256-wide tiles, one wave per SIMD
+    return p.csr.sub_block ? launch_bwd_td<T, 256, true, true>(p, ws, ws_bytes, stream)
+                           : launch_bwd_td<T, 256, true, false>(p, ws, ws_bytes, stream);
   if (p.csr.sub_block) {  // entries carry a bit mask over the pattern's 16- or 32-token blocks
     if (p.D == 128) return launch_bwd_td<T, 128, false, true>(p, ws, ws_bytes, stream);
     if (p.D == 64) return launch_bwd_td<T, 64, false, true>(p, ws, ws_bytes, stream);

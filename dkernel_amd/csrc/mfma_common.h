@@ -20,10 +20,11 @@
 
 namespace dk {
 
-// Head dims the MFMA kernels take: multiples of 8 up to 128.  They run at a
-// tile width of 64 or 128; narrower rows are zero-padded on chip.
-__host__ __device__ inline bool mfma_head_dim_ok(int d) { return d >= 8 && d <= 128 && d % 8 == 0; }
-__host__ __device__ inline int mfma_tile_width(int d) { return d <= 64 ? 64 : 128; }
+// Head dims the MFMA kernels take: multiples of 8 up to 256.  They run at a
+// tile width of 64, 128 or 256; narrower rows are zero-padded on chip.  (The
+// split-KV decode kernels stop at 128.)
+__host__ __device__ inline bool mfma_head_dim_ok(int d) { return d >= 8 && d <= 256 && d % 8 == 0; }
+__host__ __device__ inline int mfma_tile_width(int d) { return d <= 64 ? 64 : d <= 128 ? 128 : 256; }
 
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
@@ -119,7 +120,7 @@ struct Tile {
   static constexpr int kBytes = 64 * kRowBytes;
   static constexpr int kChunksPerRow = D / 8;
   static __device__ __forceinline__ int swz(int row) {
-    if constexpr (D == 128)
+    if constexpr (D >= 128)
       return ((row & 3) << 2) | ((row >> 2) & 3);
     else
       return (((row >> 1) & 1) << 2) | ((row >> 2) & 3);

@@ -37,10 +37,12 @@ struct FwdSmem {  // one stage = K tile + V tile, swizzled row-major (mfma_commo
   static constexpr int kStage = 2 * Tile<D>::kBytes;
 };
 
+// At the 256-wide tile (head dims above 128) a wave needs more than 256 registers: one wave per
+// SIMD, workgroups of at most two heads.
 // At the 64-wide tile a wave needs ~150 registers, so three waves fit a SIMD (three 4-wave
 // workgroups per CU): the softmax of one wave then has two others to hide behind.
 template <typename T, int D, int G, bool PAD, bool RP, bool SUB = false>
-__global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 ? 1 : 2, D == 64 ? 3 : 2))) void mfma_fwd_kernel(const FwdParams p, int tiles_y) {
+__global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 || D == 256 ? 1 : 2, D == 64 ? 3 : D == 256 ? 1 : 2))) void mfma_fwd_kernel(const FwdParams p, int tiles_y) {
   using M = Mma<T>;
   using vec8 = typename M::vec8;
   using S = FwdSmem<D>;
@@ -240,7 +242,24 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
     // multiply the previous batch": left alone, the compiler sinks every read
     // next to its MFMA and each multiply then waits out the LDS latency.
     vec8 va[2][DT];
-    {
+    if constexpr (D == 256) {
+      // 256-wide tiles: the K operands of a 32-key tile are fetched in two batches of eight, so
+      // that they fit the register file next to the 128 accumulator registers
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int kb = 0; kb < KS; kb += 8) {
+          vec8 ka[8];
+#pragma unroll
+          for (int i = 0; i < 8; ++i) ka[i] = lds_read8<vec8>(rd[kb + i] + ks_ + nt * 32 * TL::kRowBytes);
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) sacc[nt] = M::mma(ka[i], qf[kb + i], sacc[nt]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) va[0][dt] = lds_read_tr8<vec8>(tr[dt][0] + vs_, tr[dt][1] + vs_);
+    } else {
       vec8 ka[2][KS];
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) ka[0][ks] = lds_read8<vec8>(rd[ks] + ks_);
@@ -652,6 +671,15 @@ DK_INSTANTIATE_FWD_SUB(bf16_t, 64, true)
 DK_INSTANTIATE_FWD_SUB(f16_t, 128, true)
 DK_INSTANTIATE_FWD_SUB(f16_t, 64, true)
 #undef DK_INSTANTIATE_FWD_SUB
+// 256-wide tiles: the zero-padding instantiation only (it also takes head_dim 256 itself)
+#define DK_INSTANTIATE_FWD_256(T)                                                            \
+  template __global__ void mfma_fwd_kernel<T, 256, 1, true, false, false>(const FwdParams, int); \
+  template __global__ void mfma_fwd_kernel<T, 256, 2, true, false, false>(const FwdParams, int); \
+  template __global__ void mfma_fwd_kernel<T, 256, 2, true, true, false>(const FwdParams, int);  \
+  template __global__ void mfma_fwd_kernel<T, 256, 1, true, false, true>(const FwdParams, int);
+DK_INSTANTIATE_FWD_256(bf16_t)
+DK_INSTANTIATE_FWD_256(f16_t)
+#undef DK_INSTANTIATE_FWD_256
 DK_INSTANTIATE_FWD(bf16_t, 128, false)
 DK_INSTANTIATE_FWD(bf16_t, 64, false)
 DK_INSTANTIATE_FWD(f16_t, 128, false)
@@ -792,9 +820,34 @@ static int launch_sub(const FwdParams &p, dim3 grid, int tiles_y, hipStream_t st
   }
 }
 
+// Head dims above 128: 256-wide tiles, one or two heads per workgroup, plain or sub-block-masked
+// tables.
+template <typename T, int G, bool SUB>
+static int launch_256_g(const FwdParams &p, dim3 grid, int tiles_y, hipStream_t stream) {
+  constexpr int smem = 2 * FwdSmem<256>::kStage;
+  DK_ALLOW_DYNAMIC_LDS((mfma_fwd_kernel<T, 256, G, true, false, SUB>), smem);
+  grid.x = p.Hq / G;
+  if (int rc = launch_item_offsets(p, false, stream)) return rc;
+  hipLaunchKernelGGL((mfma_fwd_kernel<T, 256, G, true, false, SUB>), grid, dim3(128 * G), smem, stream, p, tiles_y);
+  DK_HIP_CHECK(hipGetLastError());
+  return DK_OK;
+}
+
+template <typename T>
+static int launch_256(const FwdParams &p, dim3 grid, int tiles_y, hipStream_t stream) {
+  const bool two = fwd_group(p) >= 2;
+  if (p.csr.sub_block)  // (with the mask registers two heads per workgroup would spill)
+    return launch_256_g<T, 1, true>(p, grid, tiles_y, stream);
+  // one head per workgroup: two adjacent q tiles share the workgroup and their K/V tiles
+  static const bool row_pairs = !(getenv("DKERNEL_FWD_ROWPAIR") && atoi(getenv("DKERNEL_FWD_ROWPAIR")) == 0);
+  if (!two && row_pairs) return launch_row_pairs<T, 256, true>(p, stream);
+  return two ? launch_256_g<T, 2, false>(p, grid, tiles_y, stream) : launch_256_g<T, 1, false>(p, grid, tiles_y, stream);
+}
+
 // head dims below the tile width (64 or 128) run the zero-padded instantiation
 template <typename T>
 static int launch_t(const FwdParams &p, dim3 grid, int tiles_y, hipStream_t stream) {
+  if (p.D > 128) return launch_256<T>(p, grid, tiles_y, stream);
   if (p.csr.sub_block) {  // entries carry a bit mask over the pattern's 16- or 32-token blocks
     if (p.D == 128) return launch_sub<T, 128, false>(p, grid, tiles_y, stream);
     if (p.D == 64) return launch_sub<T, 64, false>(p, grid, tiles_y, stream);

@@ -38,12 +38,12 @@ def set_impl(name: str) -> None:
 
 def _matrix_core_applies(*xs: Optional[Tensor]) -> bool:
     """Whether dk_fwd / dk_bwd will run these tensors on the matrix-core kernels with a masked tile table:
-    16-bit floats, head_dim a multiple of 8 up to 128, 16-byte aligned rows (the library's own
+    16-bit floats, head_dim a multiple of 8 up to 256, 16-byte aligned rows (the library's own
     conditions; it fails loudly if they were judged wrong here)."""
     q = xs[0]
     if _impl == _lib.DK_IMPL_GENERIC or q.dtype not in (torch.bfloat16, torch.float16):
         return False
-    if q.size(-1) % 8 or not 8 <= q.size(-1) <= 128:
+    if q.size(-1) % 8 or not 8 <= q.size(-1) <= 256:
         return False
     for x in xs:
         if x is None:

@@ -154,3 +154,33 @@ def test_backward_with_more_keys_than_queries(impl, past, Hq, Hkv, D, dtype):
     assert_close("dV", vd.grad, vo.grad, **TOL)
     assert_close("dK", kd.grad, ko.grad, **TOL)
     assert_close("dQ", qd.grad, qo.grad, **TOL)
+
+
+@pytest.mark.parametrize("D,bs,Hq,Hkv,dtype", [(256, 32, 4, 4, torch.bfloat16), (160, 64, 2, 2, torch.bfloat16),
+                                               (192, 64, 4, 2, torch.float16), (256, 64, 4, 1, torch.bfloat16),
+                                               (200, 16, 2, 2, torch.bfloat16), (136, 128, 2, 2, torch.float16)])
+def test_head_dims_above_128_on_the_matrix_cores(D, bs, Hq, Hkv, dtype):
+    """Head dims 136 ... 256 run at the 256-wide tile of the matrix-core kernels (forward, dQ,
+    dK/dV), with plain, split (blocks of 128) and sub-block-masked (blocks of 16 / 32) tables;
+    `mfma` makes the library fail instead of falling back to the generic kernels."""
+    B, L = 2, 333
+    sm = 1 / math.sqrt(D)
+    q, k, v, do = make_qkv(B, L, L, Hq, Hkv, D, dtype, with_do=True)
+    Lr = ((L + max(bs, 64) - 1) // max(bs, 64)) * max(bs, 64)
+    bm = expand_heads(OL.block_mask(Hq, Lr, bs, 2, 3, num_kv_heads=Hkv), Hq)
+    qo, ko, vo = (x.float().requires_grad_() for x in (q, k, v))
+    ro, rl = oracle_fwd(qo, ko, vo, bm, bs, sm)
+    ro.backward(do.float())
+    ops.set_impl("mfma")
+    try:
+        mod = LocalStrideSparseAttention(Hq, L, bs, 2, 3, num_kv_heads=Hkv).to(DEV)
+        qd, kd, vd = (x.to(DEV).requires_grad_() for x in (q, k, v))
+        out, lse = mod(qd, kd, vd, sm, return_lse=True)
+        out.backward(do.to(DEV))
+    finally:
+        ops.set_impl("auto")
+    assert_close("O", out, ro, **TOL)
+    assert_close("LSE", lse, rl, atol=LSE_TOL, rtol=0)
+    assert_close("dV", vd.grad, vo.grad, **TOL)
+    assert_close("dK", kd.grad, ko.grad, **TOL)
+    assert_close("dQ", qd.grad, qo.grad, **TOL)

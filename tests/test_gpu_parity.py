@@ -130,8 +130,10 @@ def test_matrix_core_kernels_take_padded_dims_and_split_blocks():
         run_fwd_bwd(1, 4, 4, 777, 40, torch.float16, 32, 3, 3)
         run_fwd_bwd(1, 4, 1, 640, 120, torch.bfloat16, 32, 2, 5)
         run_fwd_bwd(1, 2, 2, 512, 80, torch.float16, 16, 3, 9, causal=False)
+        # head dims above 128 run at the 256-wide tile
+        run_fwd_bwd(1, 2, 2, 256, 160, torch.bfloat16, 64, 2, 4)
         with pytest.raises(Exception, match="no MFMA"):
-            run_fwd_bwd(1, 2, 2, 256, 160, torch.bfloat16, 64, 2, 4)
+            run_fwd_bwd(1, 2, 2, 256, 100, torch.bfloat16, 64, 2, 4)   # not a multiple of 8
     finally:
         ops.set_impl("auto")
 

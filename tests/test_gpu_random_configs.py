@@ -26,7 +26,7 @@ def draw_config(rng):
     Hkv = int(rng.choice([1, 2, 3]))
     Hq = Hkv * ratio
     bs = int(rng.choice([64, 64, 64, 128, 256, 16, 32]))
-    D = int(rng.choice([128, 128, 64, 96, 48, 80, 112, 32]))
+    D = int(rng.choice([128, 128, 64, 96, 48, 80, 112, 32, 160, 256]))
     nb = int(rng.integers(1, 13)) if bs <= 64 else int(rng.integers(1, 6))
     L = int(rng.integers((nb - 1) * max(bs, 64) + 1, nb * max(bs, 64) + 1))
     past = int(rng.choice([0, 0, 0, 64, 37, 200])) if L > 1 else 0
@@ -144,10 +144,12 @@ def test_random_inference_config_matches_generic_kernels_and_oracle(seed):
     Hkv = int(rng.choice([1, 2]))
     Hq = Hkv * ratio
     bs = int(rng.choice([64, 64, 128, 16, 32]))
-    D = int(rng.choice([128, 64, 96, 40]))
+    D = int(rng.choice([128, 64, 96, 40, 192]))
     dtype = torch.bfloat16 if rng.random() < 0.7 else torch.float16
     mode = str(rng.choice(["left", "right", "packed", "packed_decode", "left_decode", "right_decode", "chunked",
                            "paged_decode"]))
+    if mode == "paged_decode" and D > 128:
+        D = 128    # paged K/V is served by the split-KV decode kernels, which stop at head_dim 128
     nseq = int(rng.integers(1, 6))
     Lmax = int(rng.choice([256, 512, 1024]))
     lens = [int(rng.integers(1, Lmax + 1)) for _ in range(nseq)]

@@ -23,6 +23,13 @@ from .utils import (dense_to_ccol_row, dense_to_crow_col, get_sparse_attn_mask, 
 _KERNEL_TILE = 64  # q and k tile of the matrix-core kernels
 
 
+class _NoGradContext:
+    """Stands in for the autograd context when no input requires grad."""
+
+    def save_for_backward(self, *tensors):
+        pass
+
+
 def _identical_head_run(pattern: Tensor) -> int:
     """Largest g dividing the number of pattern heads such that every run of g
     consecutive heads holds one and the same pattern."""
@@ -249,9 +256,18 @@ class SparseAttention(torch.nn.Module):
                                          self.mask_tile, self.block_size),
                                         (self.masked_csc_ccol, self.masked_csc_row, self.mask_tile,
                                          self.mask_tile, self.block_size), self.mask_lut_max_row)
-        output, lse = _sparse_attention.apply(
-            q, k, v, sm_scale, layout_csr, layout_csc,
-            self.seq_dim, inf_kwargs, kwargs)
+        needs_grad = torch.is_grad_enabled() and any(
+            x is not None and x.requires_grad for x in (q, k, v))
+        if needs_grad:
+            output, lse = _sparse_attention.apply(
+                q, k, v, sm_scale, layout_csr, layout_csc,
+                self.seq_dim, inf_kwargs, kwargs)
+        else:
+            # nothing to differentiate: the same forward without the autograd bookkeeping (several
+            # microseconds of a decode step's host time)
+            output, lse = _sparse_attention.forward(
+                _NoGradContext(), q, k, v, sm_scale, layout_csr, layout_csc,
+                self.seq_dim, inf_kwargs, kwargs)
         if return_lse:
             return output, lse
         return output

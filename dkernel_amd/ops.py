@@ -83,7 +83,23 @@ def _rowvec(x: Optional[Tensor], strides=None) -> _lib.RowVec:
     return _lib.RowVec(x.data_ptr(), sb, sh, st)
 
 
+_LUT_CACHE = {}
+
+
 def _lut(layout: Tuple[Tensor, Tensor, int, int], device, group: int = 1, max_row: int = 0) -> _lib.Lut:
+    """dk_lut of a layout tuple.  The descriptor of a module's tables never changes, so it is
+    built once per (tables, hints) and copied from then on (a decode step's host time counts)."""
+    key = (layout[0].data_ptr(), layout[1].data_ptr(), layout[0].shape, layout[1].shape, layout[0].stride(),
+           layout[1].stride(), tuple(int(x) for x in layout[2:]), device, group, max_row)
+    hit = _LUT_CACHE.get(key)
+    if hit is None:
+        if len(_LUT_CACHE) > 256:
+            _LUT_CACHE.clear()
+        hit = _LUT_CACHE[key] = _make_lut(layout, device, group, max_row)
+    return hit
+
+
+def _make_lut(layout: Tuple[Tensor, Tensor, int, int], device, group: int = 1, max_row: int = 0) -> _lib.Lut:
     ptr, idx, block_rows, block_cols = layout[:4]
     sub_block = int(layout[4]) if len(layout) > 4 else 0  # entries carry a bit mask over pattern blocks
     assert ptr.dtype == torch.int32 and idx.dtype == torch.int32
@@ -128,7 +144,16 @@ def _check_out(out: Optional[Tensor], q: Tensor) -> None:
 
 
 def _stream() -> C.c_void_p:
-    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    # the raw handle of torch's current stream (building a torch.cuda.Stream object for it costs
+    # several microseconds per call, a fifth of a decode step's host time)
+    return C.c_void_p(torch._C._cuda_getCurrentRawStream(torch.cuda.current_device()))
+
+
+def _as_i32(x: Tensor, device) -> Tensor:
+    """int32, contiguous, on `device` -- without a dispatcher round trip when it already is."""
+    if x.dtype == torch.int32 and x.device == device and x.is_contiguous():
+        return x
+    return x.to(device, dtype=torch.int32).contiguous()
 
 
 last_fwd_workspace_bytes = 0  # scratch the library asked for in the latest forward (non-zero: split-KV decode)
@@ -292,12 +317,12 @@ def padded_sparse_attn(q: Tensor, k: Tensor, v: Tensor, sm_scale: float,
 
     if left_paddings is not None:
         assert left_paddings.shape == (batches,)
-        k_starts = left_paddings.to(dev, dtype=torch.int32).contiguous()
+        k_starts = _as_i32(left_paddings, dev)
     else:
         k_starts = _const_i32(dev, batches, 0)
     if seqlens is not None:
         # ends beyond the padded length are clamped on the device
-        k_ends = k_starts + seqlens.to(dev, dtype=torch.int32)
+        k_ends = k_starts + _as_i32(seqlens, dev)
     else:
         k_ends = _const_i32(dev, batches, k_len)
     if q_len == 1:

@@ -29,10 +29,10 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16, vendor figure
 HBM_PEAK_GBS = 8000.0            # MI355X HBM3E, vendor figure
 # HBM bytes per launch, from rocprofv3 --pmc runs of this file (FETCH_SIZE scaled by the copy
 # calibration + WRITE_SIZE; profiles/fwd_bwd_decode_counters.md).  Counters cannot be read from
-# inside this process, so these are quoted, not measured live; None where no counter run exists.
+# inside this process, so these are quoted, not measured live.
 TRAFFIC_BYTES = {
     "fwd": 231.5e6 + 136.3e6,
-    "bwd": None,
+    "bwd": (621.9e6 + 68.2e6) + (641.0e6 + 134.2e6),   # dQ pass + dK/dV pass
     "decode": 180.5e6 + 0.3e6,
 }
 BS, LOCAL, VERT, D = 64, 16, 8, 128

@@ -1,5 +1,5 @@
-// MFMA backward kernels for gfx950: bf16 / fp16, head_dim 64 or 128, 64 x 64
-// blocks, equal-length unpadded sequences.  Two passes, no atomics:
+// MFMA backward kernels for gfx950: bf16 / fp16, head dims up to 256 (tiles of 64, 128 or
+// 256 columns), 64 x 64 blocks, equal-length unpadded sequences.  Two passes, no atomics:
 //
 //   dQ pass    (CSR rows)    workgroup = 64 q rows x one q head, 4 waves = 2 row
 //              halves x 2 key halves (2 waves per SIMD; the key halves are
@@ -11,13 +11,15 @@
 //              delta = rowsum(O * dO) - dLSE of its rows and leaves it in
 //              memory for the dK/dV pass, which therefore runs second.
 //   dK/dV pass (CSC columns) workgroup = 64 keys x one kv head (the q heads of
-//              a GQA group are looped inside), 8 waves: every 32 x 32 quadrant
-//              (q-row half x key half) has an S wave (S = Q K^T, P, dV^T +=
-//              dO^T P; K fragments in registers) and a dP wave (dP = dO V^T,
-//              dS = P (dP - delta), dK^T += Q^T dS; V fragments in registers).
-//              P / dS feed the second products from registers, dO^T / Q^T
-//              come from LDS transpose reads.  The two q-row halves are summed
-//              through LDS at the end.
+//              a GQA group are looped inside), 4 waves, two workgroups per
+//              CU.  A listed q block is worked on in two steps of 32 q rows;
+//              each 32 x 32 quadrant (q rows of the step x key half) has an S
+//              wave (S = Q K^T, P, dV^T += dO^T P; K fragments in registers)
+//              and a dP wave (dP = dO V^T, dS = P (dP - delta), dK^T += Q^T dS;
+//              V fragments in registers).  P / dS feed the second products
+//              from registers, dO^T / Q^T come from LDS transpose reads.
+//              Every wave owns the whole accumulator of one matrix for its 32
+//              keys, so nothing is summed across waves at the end.
 //
 // Tiles are copied HBM -> LDS asynchronously (LDS DMA, no staging registers)
 // into rings of stages, in the swizzled row-major layout of mfma_common.h.

@@ -1,4 +1,4 @@
-// MFMA forward kernel for gfx950: bf16 / fp16, head_dim 64 or 128, 64 x 64
+// MFMA forward kernel for gfx950: bf16 / fp16, head dims up to 256 (tiles of 64, 128 or 256 columns), 64 x 64
 // blocks.  Online-softmax attention over the K/V blocks listed in the CSR
 // look-up table, with LSE.
 //

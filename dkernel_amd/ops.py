@@ -12,6 +12,7 @@ synchronises with the host.
 from __future__ import annotations
 
 import ctypes as C
+import os
 import math
 from typing import Dict, Optional, Tuple, Union
 
@@ -376,6 +377,15 @@ def paged_decode_attn(q: Tensor, k_pool: Tensor, v_pool: Tensor, block_table: Te
     q4, k_pool, v_pool = _unit_last(q4), _unit_last(k_pool), _unit_last(v_pool)
     table = block_table.to(dev, dtype=torch.int32)
     table = table if table.stride(1) == 1 else table.contiguous()
+    if os.environ.get("DKERNEL_DEBUG"):
+        # The kernel cannot check page numbers against the pools' size.  This check costs a
+        # device-to-host synchronisation, so it only runs when asked for: every table entry that
+        # a sequence's tokens reach must name a page of the pools.
+        used = (torch.arange(table.size(1), device=dev)[None] * page_size) < context_lens.to(dev)[:, None]
+        bad = used & ((table < 0) | (table >= k_pool.size(0)))
+        assert not bool(bad.any()), (
+            f"block_table names pages outside the pools ({k_pool.size(0)} pages) inside a sequence: "
+            f"first at (sequence, entry) {tuple(bad.nonzero()[0].tolist())}")
     o4 = (out[:, None] if out.dim() == 3 else out) if out is not None else q4.new_empty(q4.shape)
     lse = torch.full((batches, num_heads, 1), float("-inf"), dtype=torch.float32, device=dev) if return_lse else None
     k_ends = context_lens.to(dev, dtype=torch.int32).contiguous()

@@ -88,3 +88,26 @@ def test_paged_decode_with_units_of_more_than_16_entries(page_size):
         ro, rl = _oracle(q[i:i + 1], ks[i], vs[i], bm, l, sm)
         assert_close(f"O[{i}]", out[i:i + 1, None], ro, **TOL)
         assert_close(f"LSE[{i}]", lse[i:i + 1], rl, atol=LSE_TOL, rtol=0)
+
+
+def test_debug_mode_rejects_page_numbers_outside_the_pools(monkeypatch):
+    """DKERNEL_DEBUG=1: a table entry inside a sequence that names no page of the pools is refused
+    on the host, before anything is launched (the kernel itself cannot check the upper bound)."""
+    B, Hq, Hkv, D, Lmax, ps = 2, 8, 2, 128, 1024, 64
+    g = torch.Generator().manual_seed(3)
+    q = torch.randn(B, Hq, D, generator=g).to(torch.bfloat16).to(DEV)
+    k_pool = torch.randn(40, ps, Hkv, D, generator=g).to(torch.bfloat16).to(DEV)
+    v_pool = torch.randn(40, ps, Hkv, D, generator=g).to(torch.bfloat16).to(DEV)
+    table = torch.arange(B * (Lmax // ps), dtype=torch.int32).view(B, -1)
+    lens = torch.tensor([1000, 300], dtype=torch.int32)
+    mod = LocalStrideSparseAttention.__wrapped__(Hq, Lmax, 64, 4, 2, num_kv_heads=Hkv).to(DEV)
+    monkeypatch.setenv("DKERNEL_DEBUG", "1")
+    good = mod.paged_decode(q, k_pool, v_pool, table.to(DEV), lens.to(DEV), 1 / math.sqrt(D))
+    assert torch.isfinite(good.float()).all()
+    bad = table.clone()
+    bad[1, 4] = 40        # tokens 256..319 of sequence 1 (300 keys): inside the sequence, beyond the pools
+    with pytest.raises(AssertionError, match="outside the pools"):
+        mod.paged_decode(q, k_pool, v_pool, bad.to(DEV), lens.to(DEV), 1 / math.sqrt(D))
+    bad = table.clone()
+    bad[1, 5] = 4000      # tokens 320..: beyond sequence 1's keys, never read, so not an error
+    mod.paged_decode(q, k_pool, v_pool, bad.to(DEV), lens.to(DEV), 1 / math.sqrt(D))

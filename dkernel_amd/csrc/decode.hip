@@ -206,6 +206,9 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(2, 2))) 
       // the half block's 32 keys lie in one page, or in two pages of 16
       const int psl = p.paged.page_shift, half = hb & 1;
       const int s_lo = psl < 6 ? (half * 32) >> psl : 0, s_hi = psl < 6 ? (half * 32 + 16) >> psl : 0;
+      // (lane-indexed reads: the compiler may route the lane number through M0.  Nothing in this
+      // file writes M0 behind its back - the LDS DMA helpers of mfma_common.h, which do, are not
+      // used by the decode kernels.)
       pg_lo = __builtin_amdgcn_readlane(my_page, (((hb >> 1) & 15) * 4 + s_lo) & 63);
       pg_hi = __builtin_amdgcn_readlane(my_page, (((hb >> 1) & 15) * 4 + s_hi) & 63);
       in_page0 = key0 & ((1 << psl) - 1);

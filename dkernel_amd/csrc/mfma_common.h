@@ -163,7 +163,10 @@ __device__ __forceinline__ uint32_t lds_address(const void *p) {
 }
 // M0 (the LDS base of the copy) is written without telling the compiler: it
 // rejects M0 as a clobber, and nothing else in these kernels uses M0 (on gfx950
-// only LDS DMA, lane-indexed moves and messages read it).
+// only LDS DMA, lane-indexed moves and messages read it).  Invariant for every
+// kernel that calls these helpers: no v_readlane / v_writelane / v_movrel with a
+// run-time lane or register index, and no s_sendmsg, anywhere in the kernel
+// (readfirstlane and DPP / permute exchanges do not touch M0).
 __device__ __forceinline__ uint64_t uniform_address(const void *p) {
   // the builtin returns a signed int: narrow to 32 unsigned bits before widening
   const uint64_t a = (uint64_t)p;

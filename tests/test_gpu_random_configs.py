@@ -9,6 +9,8 @@ parameters, dense heads, bf16 / fp16, token or head major layout, forward and
 backward with and without a gradient through LSE."""
 import math
 
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -18,6 +20,9 @@ from oracle import layout as OL
 from helpers import LSE_TOL, TOL, assert_close, expand_heads, oracle_fwd
 
 pytestmark = pytest.mark.gpu
+
+# DKERNEL_TEST_EXTRA_SEEDS=N appends N more seeds to every random test below (longer soak runs)
+EXTRA_SEEDS = int(os.environ.get("DKERNEL_TEST_EXTRA_SEEDS", "0"))
 DEV = "cuda"
 
 
@@ -75,7 +80,7 @@ def run_impl(impl, mod, q, k, v, do, dlse, sm, backward, sliced=False, seq_dim=1
         ops.set_impl("auto")
 
 
-@pytest.mark.parametrize("seed", range(60))
+@pytest.mark.parametrize("seed", range(60 + EXTRA_SEEDS))
 def test_random_config_matches_generic_kernels_and_oracle(seed):
     rng = np.random.default_rng(1000 + seed)
     c = draw_config(rng)
@@ -135,7 +140,7 @@ def _seq_oracle(q, k, v, bm, bs, sm):
     return o[0], lse[0]
 
 
-@pytest.mark.parametrize("seed", range(40))
+@pytest.mark.parametrize("seed", range(40 + EXTRA_SEEDS))
 def test_random_inference_config_matches_generic_kernels_and_oracle(seed):
     """Per-sequence lengths: left-padded, right-padded and packed prefill, padded, packed and
     paged single-token decode (split-KV kernels), chunked packed prefill."""
@@ -243,7 +248,7 @@ def test_random_inference_config_matches_generic_kernels_and_oracle(seed):
         assert_close(f"LSE[{i}] vs oracle", got[i][1], rl, atol=LSE_TOL, rtol=0)
 
 
-@pytest.mark.parametrize("seed", range(30))
+@pytest.mark.parametrize("seed", range(30 + EXTRA_SEEDS))
 def test_random_user_pattern_matches_generic_kernels_and_oracle(seed):
     """User-defined per-head patterns (Bernoulli blocks, diagonal forced; causal or bidirectional)
     at every block size, forward and backward: rows that share few columns, empty rows in a

@@ -77,23 +77,34 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 
     __syncthreads();
   }
 
-  // Row data of this lane (Q, dO, O fragments, lse, dLSE) is requested before anything else, so
-  // that its round trip overlaps with the table reads and the first tile request; it is used
-  // only after that request has gone out.
-  uint4 qraw[KS], doraw[KS], oraw[KS];
+  // Row data.  Q and dO of the 64 rows come in as two tiles by LDS DMA, into the second K/V stage
+  // (free until the loop's first step requests the second block), and the waves take their
+  // fragments from there: whole cache lines, fetched once for both key halves.  Loaded straight
+  // into the fragment layout (lane = row), every load instruction touches 32 rows with 32 bytes
+  // each - 96 such loads per workgroup kept the memory pipeline busy for a fifth of a short
+  // row's time.  O is only needed for delta = rowsum(O * dO) - dLSE: each thread loads four
+  // 16-byte chunks of it, consecutive lanes along a row, multiplies them with the dO chunks in
+  // LDS and the lanes of a row add up.
+  constexpr int CPR = D / 8;  // 16-byte chunks per row
+  __shared__ float delta_rows[64];
   float lse_raw = -INFINITY, dlse_raw = 0.f;
+  uint4 oreg[64 * CPR / NT];
   {
-    const T *qp = (const T *)p.q.ptr + sq.b * p.q.sb + h * p.q.sh + (int64_t)qi * p.q.st;
-    const T *dop = (const T *)p.dout.ptr + sq.b * p.dout.sb + h * p.dout.sh + (int64_t)qi * p.dout.st;
-    const T *op = (const T *)p.o.ptr + sq.b * p.o.sb + h * p.o.sh + (int64_t)qi * p.o.st;
+    const int qi0 = rb * 64 - sq.past;  // query index of the tile's first row
+    TileLoader<D, NT, PAD> qload, doload;
+    qload.init(tid, p.q.st, p.D);
+    doload.init(tid, p.dout.st, p.D);
+    const T *qb = (const T *)p.q.ptr + sq.b * p.q.sb + h * p.q.sh + (int64_t)qi0 * p.q.st;
+    const T *dob = (const T *)p.dout.ptr + sq.b * p.dout.sb + h * p.dout.sh + (int64_t)qi0 * p.dout.st;
+    qload.issue(reinterpret_cast<const char *>(qb), -qi0, sq.q_len - qi0, smem + STAGE);
+    doload.issue(reinterpret_cast<const char *>(dob), -qi0, sq.q_len - qi0, smem + STAGE + TL::kBytes);
+    const T *ob = (const T *)p.o.ptr + sq.b * p.o.sb + h * p.o.sh + (int64_t)qi0 * p.o.st;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      qraw[ks] = doraw[ks] = oraw[ks] = make_uint4(0, 0, 0, 0);
-      if (row_ok && (!PAD || ks * 16 + g * 8 < p.D)) {
-        qraw[ks] = *reinterpret_cast<const uint4 *>(qp + ks * 16 + g * 8);
-        doraw[ks] = *reinterpret_cast<const uint4 *>(dop + ks * 16 + g * 8);
-        oraw[ks] = *reinterpret_cast<const uint4 *>(op + ks * 16 + g * 8);
-      }
+    for (int j = 0; j < 64 * CPR / NT; ++j) {
+      const int r = tid / CPR + j * (NT / CPR), ch = tid % CPR;
+      oreg[j] = make_uint4(0, 0, 0, 0);
+      if (qi0 + r >= 0 && qi0 + r < sq.q_len && (!PAD || ch * 8 < p.D))
+        oreg[j] = *reinterpret_cast<const uint4 *>(ob + (int64_t)r * p.o.st + ch * 8);
     }
     if (row_ok) {
       lse_raw = p.lse.ptr[sq.b * p.lse.sb + h * p.lse.sh + (int64_t)qi * p.lse.st];
@@ -156,18 +167,28 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 
 
   // Q and dO fragments, lse in the log2 domain, and delta = rowsum(O * dO) - dLSE, which this
   // kernel computes itself and also leaves in p.delta for the dK/dV pass that follows
+  wait_tile_loads();
+  __syncthreads();  // the Q and dO tiles (and the first K/V tiles) are visible
   vec8 qf[KS], dof[KS];
-  float lse2 = INFINITY, delta = 0.f;
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) {
-    qf[ks] = as_vec8<vec8>(qraw[ks]);
-    dof[ks] = as_vec8<vec8>(doraw[ks]);
-    delta = dot8<T>(oraw[ks], doraw[ks], delta);
+    qf[ks] = lds_read8<vec8>(smem + STAGE + TL::off(rh * 32 + m, 2 * ks + g));
+    dof[ks] = lds_read8<vec8>(smem + STAGE + TL::kBytes + TL::off(rh * 32 + m, 2 * ks + g));
   }
-  delta += xor32(delta);  // the two half-waves hold the two halves of the row's head dims
+#pragma unroll
+  for (int j = 0; j < 64 * CPR / NT; ++j) {
+    const int r = tid / CPR + j * (NT / CPR), ch = tid % CPR;
+    const uint4 dow = *reinterpret_cast<const uint4 *>(smem + STAGE + TL::kBytes + TL::off(r, ch));
+    float d = dot8<T>(oreg[j], dow, 0.f);
+#pragma unroll
+    for (int off = CPR / 2; off > 0; off >>= 1) d += __shfl_xor(d, off);
+    if (ch == 0) delta_rows[r] = d;
+  }
+  __syncthreads();  // the row sums are there; every wave has its fragments: the second stage is free
+  float lse2 = INFINITY, delta = 0.f;
   if (row_ok) {
     lse2 = lse_raw == -INFINITY ? INFINITY : lse_raw * kLog2e;
-    delta -= dlse_raw;
+    delta = delta_rows[rh * 32 + m] - dlse_raw;
     if (kh == 0 && g == 0) p.delta[((int64_t)sq.b * p.Hq + h) * p.seqs.max_q_len + qi] = delta;
   }
 
@@ -263,31 +284,41 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 
     if (e + 1 < e1) block_step(e + 1, IntConst<1>{});
   }
 
-  // sum the two key halves: waves with kh = 1 hand their partial to kh = 0
+  // Sum the two key halves.  Each wave finishes half of the head dims of its rows: it hands the
+  // d-tiles of the other half to its partner through LDS and adds the partner's share to its own,
+  // so that conversions and stores are spread over all four waves.
   __syncthreads();
   float *red = reinterpret_cast<float *>(smem);
-  if (kh == 1) {
+  static_assert(DT % 2 == 0, "two halves of the d-tiles");
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
+  for (int i = 0; i < DT / 2; ++i) {
+    // (kh is wave-uniform but not a compile-time constant: the accumulator is picked by a
+    // select between two fixed registers, never by a run-time index)
+    const int dt = (1 - kh) * (DT / 2) + i;  // a d-tile of the partner's half
 #pragma unroll
-      for (int r = 0; r < 16; ++r) red[((rh * DT + dt) * 16 + r) * 64 + lane] = acc[dt][r];
+    for (int r = 0; r < 16; ++r)
+      red[((rh * DT + dt) * 16 + r) * 64 + lane] = kh == 0 ? acc[DT / 2 + i][r] : acc[i][r];
   }
   __syncthreads();
-  if (kh == 1 || !row_ok) return;
+  if (!row_ok) return;
   T *dqp = (T *)p.dq.ptr + sq.b * p.dq.sb + h * p.dq.sh + (int64_t)qi * p.dq.st;
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt)
+  for (int i = 0; i < DT / 2; ++i) {
 #pragma unroll
     for (int r4 = 0; r4 < 4; ++r4) {
       T o4[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int r = r4 * 4 + i;
-        o4[i] = from_float<T>((acc[dt][r] + red[((rh * DT + dt) * 16 + r) * 64 + lane]) * p.sm_scale);
+      for (int j = 0; j < 4; ++j) {
+        const int r = r4 * 4 + j;
+        const float own = kh == 0 ? acc[i][r] : acc[DT / 2 + i][r];
+        const int dt = kh * (DT / 2) + i;
+        o4[j] = from_float<T>((own + red[((rh * DT + dt) * 16 + r) * 64 + lane]) * p.sm_scale);
       }
+      const int dt = kh * (DT / 2) + i;
       if (!PAD || dt * 32 + r4 * 8 + g * 4 < p.D)
         *reinterpret_cast<uint2 *>(dqp + dt * 32 + r4 * 8 + g * 4) = *reinterpret_cast<const uint2 *>(o4);
     }
+  }
 }
 
 // ---------------------------------------------------------------------------

@@ -382,9 +382,33 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 
   const int key = cb * 64 + nh * 32 + n;
   const bool key_ok = key < sq.k_len;
 
-  // K fragments (S wave) or V fragments (dP wave): B operand of the first product
+  Loader qload, doload;
+  qload.init(tid, p.q.st, p.D);
+  doload.init(tid, p.dout.st, p.D);
+  if constexpr (PAD) {  // the slots of the head dims beyond p.D stay zero in every stage
+    zero_tiles<NT>(smem, S::kBytes, tid);
+    __syncthreads();
+  }
+  // K fragments (S wave) or V fragments (dP wave): B operand of the first product.  Up to the
+  // 128-wide tile the K and V tiles of the column come in by LDS DMA (whole cache lines; K into
+  // the two Q stages that the first two steps do not use, V into the P exchange area) and the
+  // waves take their fragments from there behind the first tile wait.  Loaded straight into the
+  // fragment layout (lane = key), every load instruction touches 32 rows with 32 bytes each:
+  // measured 8 % of the pass on columns of 16 blocks.  (At the 256-wide tile the V tile does not
+  // fit the exchange area: direct loads.)
+  constexpr bool kKvTiles = D <= 128;
+  char *const k_tile = smem + S::kQ + 2 * S::kTile, *const v_tile = smem + S::kX;
   vec8 kvf[KS];
-  {
+  if constexpr (kKvTiles) {
+    static_assert(!kKvTiles || (2 * S::kTile == TL::kBytes && 2 * 2 * 4096 >= TL::kBytes), "a 64-row tile fits either place");
+    TileLoader<D, NT, PAD> kload, vload;
+    kload.init(tid, p.k.st, p.D);
+    vload.init(tid, p.v.st, p.D);
+    const T *kb = (const T *)p.k.ptr + sq.b * p.k.sb + kvh * p.k.sh + (int64_t)cb * 64 * p.k.st;
+    const T *vb = (const T *)p.v.ptr + sq.b * p.v.sb + kvh * p.v.sh + (int64_t)cb * 64 * p.v.st;
+    kload.issue(reinterpret_cast<const char *>(kb), 0, sq.k_len - cb * 64, k_tile);
+    vload.issue(reinterpret_cast<const char *>(vb), 0, sq.k_len - cb * 64, v_tile);
+  } else {
     const T *src = dp_wave ? (const T *)p.v.ptr + sq.b * p.v.sb + kvh * p.v.sh + (int64_t)key * p.v.st
                            : (const T *)p.k.ptr + sq.b * p.k.sb + kvh * p.k.sh + (int64_t)key * p.k.st;
 #pragma unroll
@@ -406,20 +430,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[dt][r] = 0.f;
 
-  Loader qload, doload;
-  qload.init(tid, p.q.st, p.D);
-  doload.init(tid, p.dout.st, p.D);
-  if constexpr (PAD) {  // the slots of the head dims beyond p.D stay zero in every Q / dO stage
-    zero_tiles<NT>(smem, S::kVec, tid);
-    __syncthreads();
-  }
   int rd[KS], tr[DT][2];
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) rd[ks] = TL::off(n, 2 * ks + g);
   transposed_offsets<D>(lane, tr);
   float *xbuf = reinterpret_cast<float *>(smem + S::kX) + nh * 2 * 1024;  // this pair's two P buffers
 
-  for (int gq = gq_first; gq < gq_end; ++gq) {
+  // (the body is instantiated twice: the first head also takes the K / V fragments out of LDS,
+  // unconditionally - guarded by a run-time test on gq the fragments and accumulators spill)
+  auto head_body = [&](int gq, auto first_tag) {
     const int h = kvh * ratio + gq;
     const int lh = lut_head(p.csc, h, p.Hq, p.Hkv);
     int e0 = 0, e1 = 0;
@@ -502,6 +521,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 
         exact = issue(rb_next, i, iq, ido) && exact;
         iq = iq + 1 == S::kQStages ? 0 : iq + 1;
         ido = ido + 1 == S::kDoStages ? 0 : ido + 1;
+      }
+    }
+    if constexpr (kKvTiles) {
+      if constexpr (decltype(first_tag)::value) {
+        // the K / V tiles are older than the requests above: everything has landed behind this wait
+        wait_tile_loads();
+        __syncthreads();
+        const char *src = dp_wave ? v_tile : k_tile;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) kvf[ks] = lds_read8<vec8>(src + TL::off(nh * 32 + n, 2 * ks + g));
+        // (the loop's first barrier comes before anything is copied over the two tiles: step 2's Q
+        // tile is requested behind it, and the S waves write P behind it)
       }
     }
     floatx16 dp_prev;
@@ -627,7 +658,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 
     else
       run_head(BoolConst<false>{});
     if (gq + 1 < gq_end) __syncthreads();  // every wave is done with every stage before the next head reuses them
-  }
+  };
+  head_body(gq_first, BoolConst<true>{});
+  for (int gq = gq_first + 1; gq < gq_end; ++gq) head_body(gq, BoolConst<false>{});
 
   // every wave holds the finished dV^T (S wave) or dK^T (dP wave) of its 32 keys
   if (!key_ok) return;

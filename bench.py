@@ -32,7 +32,7 @@ HBM_PEAK_GBS = 8000.0            # MI355X HBM3E, vendor figure
 # inside this process, so these are quoted, not measured live.
 TRAFFIC_BYTES = {
     "fwd": 231.5e6 + 136.3e6,
-    "bwd": (621.9e6 + 68.2e6) + (641.0e6 + 134.2e6),   # dQ pass + dK/dV pass
+    "bwd": (616.3e6 + 68.2e6) + (629.5e6 + 134.2e6),   # dQ pass + dK/dV pass
     "decode": 180.5e6 + 0.3e6,
 }
 BS, LOCAL, VERT, D = 64, 16, 8, 128

@@ -278,6 +278,49 @@ struct TileLoader {
   }
 };
 
+// Write a wave's 32 x D accumulator tile (registers hold acc^T: lane = row m, register = dim) as
+// rows of `T` scaled by `row_scale`: the tile goes through `stage` (32 rows of LDS in the tile
+// layout, owned by this wave) and leaves as 16-byte pieces, CPR consecutive lanes covering one
+// whole row, with the non-temporal hint.  Whole rows written around the L2 measure faster than
+// the 8-byte pieces a lane holds after the multiply (forward: -3 % headline, -8 % at 8 blocks
+// per row); either change alone does not (coalescing alone: no change; the hint on 8-byte
+// pieces: much slower).  Rows outside [row_lo, row_hi) are not written.  The caller makes sure
+// that no wave still reads `stage` (a barrier after the last tile read).
+template <typename T, int D, bool PAD, int ROWS>
+__device__ __forceinline__ void store_staged_rows(const char *stage, T *g_row0, int64_t row_stride, int lane,
+                                                  int row_lo, int row_hi, int real_d) {
+  // rows 0 .. ROWS-1 of `stage` (tile layout) to g_row0 + row * row_stride, by one wave
+  using TL = Tile<D>;
+  constexpr int CPR = D / 8, RPI = 64 / CPR;
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+#pragma unroll
+  for (int j = 0; j < ROWS / RPI; ++j) {
+    const int r = j * RPI + lane / CPR, c = lane % CPR;
+    const u32x4 w = *reinterpret_cast<const u32x4 *>(stage + TL::off(r, c));
+    if (r >= row_lo && r < row_hi && (!PAD || c * 8 < real_d))
+      __builtin_nontemporal_store(w, reinterpret_cast<u32x4 *>(g_row0 + (int64_t)r * row_stride + c * 8));
+  }
+}
+
+template <typename T, int D, bool PAD>
+__device__ __forceinline__ void store_tile_rows(char *stage, const floatx16 (&acc)[D / 32], float row_scale, T *g_row0,
+                                                int64_t row_stride, int lane, int row_lo, int row_hi, int real_d) {
+  using TL = Tile<D>;
+  constexpr int DT = D / 32;
+  const int m = lane & 31, g = lane >> 5;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int r4 = 0; r4 < 4; ++r4) {
+      // registers 4*r4 .. 4*r4+3 are dims 32dt + 8r4 + 4g + {0..3}
+      T o4[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o4[i] = from_float<T>(acc[dt][r4 * 4 + i] * row_scale);
+      *reinterpret_cast<uint2 *>(stage + TL::off(m, dt * 4 + r4) + g * 8) = *reinterpret_cast<const uint2 *>(o4);
+    }
+  store_staged_rows<T, D, PAD, 32>(stage, g_row0, row_stride, lane, row_lo, row_hi, real_d);
+}
+
 // Zero `bytes` (a multiple of 16) of LDS with NT threads; the caller synchronises afterwards.
 template <int NT>
 __device__ __forceinline__ void zero_tiles(char *lds, int bytes, int tid) {

@@ -371,20 +371,15 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
   l_run += xor32(l_run);
 
   // ---- epilogue: O = O^T / l, LSE = (m + log2 l) ln 2 ----
-  if (!row_ok) return;
+  __syncthreads();  // the K / V stages are free: each wave stages its O tile in 32 rows of them
   const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
-  T *op = (T *)p.o.ptr + sq.b * p.o.sb + h * p.o.sh + (int64_t)(sq.q_start + qi) * p.o.st;
-#pragma unroll
-  for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-    for (int r4 = 0; r4 < 4; ++r4) {
-      // registers 4*r4 .. 4*r4+3 are dims 32dt + 8r4 + 4g + {0..3}
-      T o4[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) o4[i] = from_float<T>(oacc[dt][r4 * 4 + i] * inv);
-      if (!PAD || dt * 32 + r4 * 8 + g * 4 < p.D)
-        *reinterpret_cast<uint2 *>(op + dt * 32 + r4 * 8 + g * 4) = *reinterpret_cast<const uint2 *>(o4);
-    }
+  {
+    const int qi0 = row0 - sq.past;  // may be negative or beyond q_len: those rows are skipped
+    T *o_row0 = (T *)p.o.ptr + sq.b * p.o.sb + h * p.o.sh + (int64_t)(sq.q_start + qi0) * p.o.st;
+    store_tile_rows<T, D, PAD>(smem + wave * 32 * TL::kRowBytes, oacc, inv, o_row0, p.o.st, lane, -qi0,
+                               sq.q_len - qi0, p.D);
+  }
+  if (!row_ok) return;
   if (p.lse.ptr && g == 0) {
     const float lse = l_run > 0.f ? (m_run + log2f(l_run)) * kLn2 : -INFINITY;
     p.lse.ptr[sq.b * p.lse.sb + h * p.lse.sh + (int64_t)(sq.q_start + qi) * p.lse.st] = lse;
@@ -631,19 +626,15 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
   }
   l_run += xor32(l_run);
 
-  if (!row_ok) return;
+  __syncthreads();  // the tile rings are free: each wave stages its O tile in 32 rows of them
   const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
-  T *op = (T *)p.o.ptr + sq.b * p.o.sb + h * p.o.sh + (int64_t)(sq.q_start + qi) * p.o.st;
-#pragma unroll
-  for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-    for (int r4 = 0; r4 < 4; ++r4) {
-      T o4[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) o4[i] = from_float<T>(oacc[dt][r4 * 4 + i] * inv);
-      if (!PAD || dt * 32 + r4 * 8 + g * 4 < p.D)
-        *reinterpret_cast<uint2 *>(op + dt * 32 + r4 * 8 + g * 4) = *reinterpret_cast<const uint2 *>(o4);
-    }
+  {
+    const int qi0 = row0 - sq.past;
+    T *o_row0 = (T *)p.o.ptr + sq.b * p.o.sb + h * p.o.sh + (int64_t)(sq.q_start + qi0) * p.o.st;
+    store_tile_rows<T, D, PAD>(smem + wave * 32 * TL::kRowBytes, oacc, inv, o_row0, p.o.st, lane, -qi0,
+                               sq.q_len - qi0, p.D);
+  }
+  if (!row_ok) return;
   if (p.lse.ptr && g == 0) {
     const float lse = l_run > 0.f ? (m_run + log2f(l_run)) * kLn2 : -INFINITY;
     p.lse.ptr[sq.b * p.lse.sb + h * p.lse.sh + (int64_t)(sq.q_start + qi) * p.lse.st] = lse;

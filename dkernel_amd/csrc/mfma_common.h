@@ -281,24 +281,39 @@ struct TileLoader {
 // Write a wave's 32 x D accumulator tile (registers hold acc^T: lane = row m, register = dim) as
 // rows of `T` scaled by `row_scale`: the tile goes through `stage` (32 rows of LDS in the tile
 // layout, owned by this wave) and leaves as 16-byte pieces, CPR consecutive lanes covering one
-// whole row, with the non-temporal hint.  Whole rows written around the L2 measure faster than
-// the 8-byte pieces a lane holds after the multiply (forward: -3 % headline, -8 % at 8 blocks
-// per row); either change alone does not (coalescing alone: no change; the hint on 8-byte
-// pieces: much slower).  Rows outside [row_lo, row_hi) are not written.  The caller makes sure
-// that no wave still reads `stage` (a barrier after the last tile read).
+// whole row, with the non-temporal hint.  Whole rows written around the L2 measure faster in
+// the forward than the 8-byte pieces a lane holds after the multiply (-3 % on the headline
+// workload, -8 % at 8 blocks per row); either change alone does not (coalescing alone: no
+// change; the hint on 8-byte pieces: much slower).  The backward kernels keep direct stores:
+// the same change measured +-0.5 % at the 128-wide tile and +1.3 % at the 64-wide one there.
+// Rows outside [row_lo, row_hi) are not written.  The caller makes sure that no wave still
+// reads `stage` (a barrier after the last tile read).
 template <typename T, int D, bool PAD, int ROWS>
 __device__ __forceinline__ void store_staged_rows(const char *stage, T *g_row0, int64_t row_stride, int lane,
                                                   int row_lo, int row_hi, int real_d) {
-  // rows 0 .. ROWS-1 of `stage` (tile layout) to g_row0 + row * row_stride, by one wave
+  // rows 0 .. ROWS-1 of `stage` (tile layout) to g_row0 + row * row_stride, by one wave.  The
+  // non-temporal hint only where every row is a run of whole 128-byte lines: on partial lines
+  // it is slower than plain stores.
   using TL = Tile<D>;
   constexpr int CPR = D / 8, RPI = 64 / CPR;
   typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  // (the lane number passes through an empty asm statement: the addresses below are then
+  // computed here, not hoisted to the start of the kernel, where they would occupy registers
+  // through the main loop)
+  asm volatile("" : "+v"(lane));
+  const bool whole_lines = __builtin_amdgcn_readfirstlane(
+      (int)(((uintptr_t)g_row0 | (uintptr_t)(row_stride * (int64_t)sizeof(T)) | (uintptr_t)(real_d * sizeof(T))) & 127) == 0);
 #pragma unroll
   for (int j = 0; j < ROWS / RPI; ++j) {
     const int r = j * RPI + lane / CPR, c = lane % CPR;
     const u32x4 w = *reinterpret_cast<const u32x4 *>(stage + TL::off(r, c));
-    if (r >= row_lo && r < row_hi && (!PAD || c * 8 < real_d))
-      __builtin_nontemporal_store(w, reinterpret_cast<u32x4 *>(g_row0 + (int64_t)r * row_stride + c * 8));
+    if (r >= row_lo && r < row_hi && (!PAD || c * 8 < real_d)) {
+      u32x4 *dst = reinterpret_cast<u32x4 *>(g_row0 + (int64_t)r * row_stride + c * 8);
+      if (whole_lines)
+        __builtin_nontemporal_store(w, dst);
+      else
+        *dst = w;
+    }
   }
 }
 
@@ -307,6 +322,7 @@ __device__ __forceinline__ void store_tile_rows(char *stage, const floatx16 (&ac
                                                 int64_t row_stride, int lane, int row_lo, int row_hi, int real_d) {
   using TL = Tile<D>;
   constexpr int DT = D / 32;
+  asm volatile("" : "+v"(lane));  // as in store_staged_rows
   const int m = lane & 31, g = lane >> 5;
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt)

@@ -300,24 +300,44 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 
       red[((rh * DT + dt) * 16 + r) * 64 + lane] = kh == 0 ? acc[DT / 2 + i][r] : acc[i][r];
   }
   __syncthreads();
-  if (!row_ok) return;
+  // From the 128-wide tile on the finished rows go through a 64-row tile behind the exchange
+  // area and leave as whole rows with the non-temporal hint (16 rows per wave): -1 % of the
+  // backward at head_dim 128, -1.5 % at 192 / 256.  At the 64-wide tile the direct 8-byte
+  // stores of the accumulator layout measure 0.5 % faster and stay.
+  constexpr bool kStagedStores = D >= 128;
+  char *const out_tile = smem + 2 * DT * 16 * 64 * (int)sizeof(float);
+  static_assert(2 * DT * 16 * 64 * (int)sizeof(float) + TL::kBytes <= 2 * STAGE, "exchange area and output tile fit the stages");
+  if constexpr (!kStagedStores) {
+    if (!row_ok) return;
+  }
+  int lane_late = lane;  // opaque copy: the tile addresses below are computed here, not before the loop
+  asm volatile("" : "+v"(lane_late));
+  const int m_late = lane_late & 31, g_late = lane_late >> 5;
   T *dqp = (T *)p.dq.ptr + sq.b * p.dq.sb + h * p.dq.sh + (int64_t)qi * p.dq.st;
 #pragma unroll
   for (int i = 0; i < DT / 2; ++i) {
 #pragma unroll
     for (int r4 = 0; r4 < 4; ++r4) {
       T o4[4];
+      const int dt = kh * (DT / 2) + i;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int r = r4 * 4 + j;
         const float own = kh == 0 ? acc[i][r] : acc[DT / 2 + i][r];
-        const int dt = kh * (DT / 2) + i;
         o4[j] = from_float<T>((own + red[((rh * DT + dt) * 16 + r) * 64 + lane]) * p.sm_scale);
       }
-      const int dt = kh * (DT / 2) + i;
-      if (!PAD || dt * 32 + r4 * 8 + g * 4 < p.D)
+      // registers 4*r4 .. 4*r4+3 are dims 32dt + 8r4 + 4g + {0..3}
+      if constexpr (kStagedStores)
+        *reinterpret_cast<uint2 *>(out_tile + TL::off(rh * 32 + m_late, dt * 4 + r4) + g_late * 8) = *reinterpret_cast<const uint2 *>(o4);
+      else if (!PAD || dt * 32 + r4 * 8 + g * 4 < p.D)
         *reinterpret_cast<uint2 *>(dqp + dt * 32 + r4 * 8 + g * 4) = *reinterpret_cast<const uint2 *>(o4);
     }
+  }
+  if constexpr (kStagedStores) {
+    __syncthreads();
+    const int qi0 = rb * 64 + wave * 16 - sq.past;  // query index of this wave's first row
+    T *dq_row0 = (T *)p.dq.ptr + sq.b * p.dq.sb + h * p.dq.sh + (int64_t)qi0 * p.dq.st;
+    store_staged_rows<T, D, PAD, 16>(out_tile + wave * 16 * TL::kRowBytes, dq_row0, p.dq.st, lane, -qi0, sq.q_len - qi0, p.D);
   }
 }
 
@@ -663,12 +683,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 
   for (int gq = gq_first + 1; gq < gq_end; ++gq) head_body(gq, BoolConst<false>{});
 
   // every wave holds the finished dV^T (S wave) or dK^T (dP wave) of its 32 keys
-  if (!key_ok) return;
   const float out_scale = dp_wave ? p.sm_scale : 1.f;
   const TensorView &outv = dp_wave ? p.dk : p.dv;
-  const int64_t out_off = sq.b * outv.sb + out_head * outv.sh + (int64_t)key * outv.st;
   if (head_split) {  // fp32 partial of this q head
-    float *outp = (float *)outv.ptr + out_off;
+    if (!key_ok) return;
+    float *outp = (float *)outv.ptr + sq.b * outv.sb + out_head * outv.sh + (int64_t)key * outv.st;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -682,17 +701,27 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 
       }
     return;
   }
-  T *outp = (T *)outv.ptr + out_off;
+  if constexpr (D >= 128) {
+    // each wave stages its 32 keys x D in one stage of the Q ring and writes whole rows (as in
+    // the dQ pass: from the 128-wide tile on)
+    __syncthreads();  // the dP waves have finished their last step (it reads the Q ring)
+    const int key0 = cb * 64 + nh * 32;
+    T *out_row0 = (T *)outv.ptr + sq.b * outv.sb + out_head * outv.sh + (int64_t)key0 * outv.st;
+    store_tile_rows<T, D, PAD>(smem + S::kQ + wave * S::kTile, acc, out_scale, out_row0, outv.st, lane, 0, sq.k_len - key0, p.D);
+  } else {
+    if (!key_ok) return;
+    T *outp = (T *)outv.ptr + sq.b * outv.sb + out_head * outv.sh + (int64_t)key * outv.st;
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt)
+    for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-    for (int r4 = 0; r4 < 4; ++r4) {
-      T o4[4];
+      for (int r4 = 0; r4 < 4; ++r4) {
+        T o4[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) o4[i] = from_float<T>(acc[dt][r4 * 4 + i] * out_scale);
-      if (!PAD || dt * 32 + r4 * 8 + g * 4 < p.D)
-        *reinterpret_cast<uint2 *>(outp + dt * 32 + r4 * 8 + g * 4) = *reinterpret_cast<const uint2 *>(o4);
-    }
+        for (int i = 0; i < 4; ++i) o4[i] = from_float<T>(acc[dt][r4 * 4 + i] * out_scale);
+        if (!PAD || dt * 32 + r4 * 8 + g * 4 < p.D)
+          *reinterpret_cast<uint2 *>(outp + dt * 32 + r4 * 8 + g * 4) = *reinterpret_cast<const uint2 *>(o4);
+      }
+  }
 }
 
 // Explicit instantiations: with only the implicit ones the fp16 host stubs of

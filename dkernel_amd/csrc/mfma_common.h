@@ -291,9 +291,7 @@ struct TileLoader {
 template <typename T, int D, bool PAD, int ROWS>
 __device__ __forceinline__ void store_staged_rows(const char *stage, T *g_row0, int64_t row_stride, int lane,
                                                   int row_lo, int row_hi, int real_d) {
-  // rows 0 .. ROWS-1 of `stage` (tile layout) to g_row0 + row * row_stride, by one wave.  The
-  // non-temporal hint only where every row is a run of whole 128-byte lines: on partial lines
-  // it is slower than plain stores.
+  // rows 0 .. ROWS-1 of `stage` (tile layout) to g_row0 + row * row_stride, by one wave
   using TL = Tile<D>;
   constexpr int CPR = D / 8, RPI = 64 / CPR;
   typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -301,19 +299,14 @@ __device__ __forceinline__ void store_staged_rows(const char *stage, T *g_row0, 
   // computed here, not hoisted to the start of the kernel, where they would occupy registers
   // through the main loop)
   asm volatile("" : "+v"(lane));
-  const bool whole_lines = __builtin_amdgcn_readfirstlane(
-      (int)(((uintptr_t)g_row0 | (uintptr_t)(row_stride * (int64_t)sizeof(T)) | (uintptr_t)(real_d * sizeof(T))) & 127) == 0);
 #pragma unroll
   for (int j = 0; j < ROWS / RPI; ++j) {
     const int r = j * RPI + lane / CPR, c = lane % CPR;
     const u32x4 w = *reinterpret_cast<const u32x4 *>(stage + TL::off(r, c));
-    if (r >= row_lo && r < row_hi && (!PAD || c * 8 < real_d)) {
-      u32x4 *dst = reinterpret_cast<u32x4 *>(g_row0 + (int64_t)r * row_stride + c * 8);
-      if (whole_lines)
-        __builtin_nontemporal_store(w, dst);
-      else
-        *dst = w;
-    }
+    // (the hint is unconditional on purpose: behind a run-time test with a plain store in the
+    // other branch the compiler merges the two stores into one plain store)
+    if (r >= row_lo && r < row_hi && (!PAD || c * 8 < real_d))
+      __builtin_nontemporal_store(w, reinterpret_cast<u32x4 *>(g_row0 + (int64_t)r * row_stride + c * 8));
   }
 }
 

@@ -126,10 +126,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 
   TileLoader<D, NT, PAD> kload, vload;
   kload.init(tid, p.k.st, p.D);
   vload.init(tid, p.v.st, p.D);
+  // blocks whose first key lies in [0, k_full_span) hold 64 keys of the sequence
+  const uint32_t k_full_span = sq.k_len >= 64 ? (uint32_t)(sq.k_len - 64) + 1u : 0u;
+  const uint32_t k_row_bytes = (uint32_t)p.k.st * 2u, v_row_bytes = (uint32_t)p.v.st * 2u;
   auto issue = [&](int col, int stage) {  // asynchronous copy of K/V block `col` into `stage`
     const int key0 = col * 64;
-    const int valid = col < 0 ? 0 : sq.k_len - key0;
     char *ks = smem + stage * STAGE;
+    if ((uint32_t)key0 < k_full_span) {  // main path (one scalar compare; a padding entry is negative)
+      kload.issue_full(row_address(reinterpret_cast<const char *>(kbase), key0, k_row_bytes), ks);
+      vload.issue_full(row_address(reinterpret_cast<const char *>(vbase), key0, v_row_bytes), ks + TL::kBytes);
+      return;
+    }
+    const int valid = col < 0 ? 0 : sq.k_len - key0;
     kload.issue(reinterpret_cast<const char *>(kbase + (int64_t)key0 * p.k.st), 0, valid, ks);
     vload.issue(reinterpret_cast<const char *>(vbase + (int64_t)key0 * p.v.st), 0, valid, ks + TL::kBytes);
   };
@@ -456,6 +464,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 
   transposed_offsets<D>(lane, tr);
   float *xbuf = reinterpret_cast<float *>(smem + S::kX) + nh * 2 * 1024;  // this pair's two P buffers
 
+  // tiles whose first query index lies in [0, full_span) hold 32 queries
+  const uint32_t full_span = sq.q_len >= S::kRows ? (uint32_t)(sq.q_len - S::kRows) + 1u : 0u;
+  const uint32_t q_row_bytes = (uint32_t)p.q.st * 2u, do_row_bytes = (uint32_t)p.dout.st * 2u;
   // (the body is instantiated twice: the first head also takes the K / V fragments out of LDS,
   // unconditionally - guarded by a run-time test on gq the fragments and accumulators spill)
   auto head_body = [&](int gq, auto first_tag) {
@@ -477,15 +488,26 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 
     // when rows had to be zero-filled, i.e. when the per-wave load count is not LPT.
     auto issue = [&](int rbq, int half, int qstage, int dostage) -> bool {
       const int qi0 = rbq * 64 + half * 32 - sq.past;  // query index of the tile's first row
+      const int row = lane & 31;
+      const bool is_delta = lane >= 32;
+      char *dst = smem + S::kVec + qstage * 256;
+      // main path: a listed block whose 32 rows all are queries (one scalar compare: a padding
+      // entry, rbq < 0, gives a negative qi0)
+      if ((uint32_t)qi0 < full_span) {
+        qload.issue_full(row_address(reinterpret_cast<const char *>(qbase), qi0, q_row_bytes),
+                         smem + S::kQ + qstage * S::kTile);
+        doload.issue_full(row_address(reinterpret_cast<const char *>(dobase), qi0, do_row_bytes),
+                          smem + S::kDo + dostage * S::kTile);
+        const float *src = is_delta ? deltabase + qi0 + row : lsebase + (int64_t)(qi0 + row) * p.lse.st;
+        lds_dma4_lane(src, lds_address(dst));
+        return true;
+      }
       // rows before the first query (qi < 0, when k is longer than q) and beyond the last are zero-filled
       const int lo = rbq < 0 ? S::kRows : -qi0, hi = sq.q_len - qi0;
       const bool full = qload.issue(reinterpret_cast<const char *>(qbase + (int64_t)qi0 * p.q.st), lo, hi,
                                     smem + S::kQ + qstage * S::kTile);
       doload.issue(reinterpret_cast<const char *>(dobase + (int64_t)qi0 * p.dout.st), lo, hi,
                    smem + S::kDo + dostage * S::kTile);
-      const int row = lane & 31;
-      const bool is_delta = lane >= 32;
-      char *dst = smem + S::kVec + qstage * 256;
       if (full) {
         const float *src = is_delta ? deltabase + qi0 + row : lsebase + (int64_t)(qi0 + row) * p.lse.st;
         lds_dma4_lane(src, lds_address(dst));
@@ -816,7 +838,8 @@ bool mfma_bwd_supported(const BwdParams &p, int dtype) {
          p.csr.block_cols == 64 && p.csr.sub_block == p.csc.sub_block &&
          (p.csr.sub_block != 0 || (p.csr.entry_width == 1 && p.csc.entry_width == 1)) &&
          p.csc.block_rows == 64 && p.csc.block_cols == 64 &&
-         p.vec_ok;
+         p.vec_ok && mfma_row_bytes_ok(p.q) && mfma_row_bytes_ok(p.k) && mfma_row_bytes_ok(p.v) &&
+         mfma_row_bytes_ok(p.dout);
 }
 
 template <typename T, int D, bool PAD, bool SUB>

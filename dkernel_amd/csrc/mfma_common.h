@@ -24,6 +24,9 @@ namespace dk {
 // tile width of 64, 128 or 256; narrower rows are zero-padded on chip.  (The
 // split-KV decode kernels stop at 128.)
 __host__ __device__ inline bool mfma_head_dim_ok(int d) { return d >= 8 && d <= 256 && d % 8 == 0; }
+// the kernels keep a row's byte stride in 32 bits (16-bit elements)
+template <typename View>
+inline bool mfma_row_bytes_ok(const View &t) { return t.st >= 0 && t.st < (int64_t(1) << 31); }
 __host__ __device__ inline int mfma_tile_width(int d) { return d <= 64 ? 64 : d <= 128 ? 128 : 256; }
 
 
@@ -190,6 +193,12 @@ __device__ __forceinline__ void scalar_load2(const int32_t *p0, const int32_t *p
                : "s"(uniform_address(p0)), "s"(uniform_address(p1))
                : "memory");
 }
+// base + rows * row_bytes for a wave-uniform, non-negative row count: one 32 x 32 -> 64 bit
+// unsigned multiply (two scalar instructions) where `base + (int64_t)rows * stride` takes a
+// signed 64 x 64 bit one (six).
+__device__ __forceinline__ const char *row_address(const char *base, int rows, uint32_t row_bytes) {
+  return base + (uint64_t)(uint32_t)rows * (uint64_t)row_bytes;
+}
 __device__ __forceinline__ void lds_dma16(const char *gbase, uint32_t voff, uint32_t lds_base) {
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                :
@@ -252,6 +261,16 @@ struct TileLoader {
       if (chunk * 8 < real_d) inside |= 1u << c;
     }
   }
+  // The whole tile lies inside the tensor: kChunks load instructions per wave and nothing else.
+  // Callers test for this case with scalar arithmetic and take it on the main path: the general
+  // `issue` below costs some thirty scalar instructions per tile in range tests and selects,
+  // which all waves of a CU execute behind the same barrier.
+  __device__ __forceinline__ void issue_full(const char *gblk, char *tile) const {
+    const uint32_t base = lds_address(tile) + row0 * Tile<D>::kRowBytes;
+#pragma unroll
+    for (int c = 0; c < kChunks; ++c)
+      if (!PAD || ((inside >> c) & 1)) lds_dma16(gblk, goff[c], base + c * (NT / kCPR) * Tile<D>::kRowBytes);
+  }
   // rows [lo, hi) of the block are copied, the others zero-filled.  Returns true when the
   // whole tile was copied, i.e. when every wave issued exactly kChunks load instructions.
   // gblk (first byte of the 64-row block) is wave-uniform.
@@ -284,8 +303,8 @@ struct TileLoader {
 // whole row, with the non-temporal hint.  Whole rows written around the L2 measure faster in
 // the forward than the 8-byte pieces a lane holds after the multiply (-3 % on the headline
 // workload, -8 % at 8 blocks per row); either change alone does not (coalescing alone: no
-// change; the hint on 8-byte pieces: much slower).  The backward kernels keep direct stores:
-// the same change measured +-0.5 % at the 128-wide tile and +1.3 % at the 64-wide one there.
+// change; the hint on 8-byte pieces: much slower).  The backward kernels use it from the
+// 128-wide tile on (-1 % there; at the 64-wide tile direct stores are 0.5 % faster).
 // Rows outside [row_lo, row_hi) are not written.  The caller makes sure that no wave still
 // reads `stage` (a barrier after the last tile read).
 template <typename T, int D, bool PAD, int ROWS>

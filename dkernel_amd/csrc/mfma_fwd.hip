@@ -135,10 +135,18 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
   TileLoader<D, NT, PAD> kload, vload;
   kload.init(tid, p.k.st, p.D);
   vload.init(tid, p.v.st, p.D);
+  // blocks whose first key lies in [0, k_full_span) hold 64 keys of the sequence
+  const uint32_t k_full_span = sq.k_len >= 64 ? (uint32_t)(sq.k_len - 64) + 1u : 0u;
+  const uint32_t k_row_bytes = (uint32_t)p.k.st * 2u, v_row_bytes = (uint32_t)p.v.st * 2u;
   auto issue = [&](int col, int stage) {
     const int key0 = col * 64;
-    const int valid = col < 0 ? 0 : sq.k_len - key0;
     char *ks = smem + stage * S::kStage;
+    if ((uint32_t)key0 < k_full_span) {  // main path (one scalar compare; a padding entry is negative)
+      kload.issue_full(row_address(reinterpret_cast<const char *>(kbase), key0, k_row_bytes), ks);
+      vload.issue_full(row_address(reinterpret_cast<const char *>(vbase), key0, v_row_bytes), ks + TL::kBytes);
+      return;
+    }
+    const int valid = col < 0 ? 0 : sq.k_len - key0;
     kload.issue(reinterpret_cast<const char *>(kbase + (int64_t)key0 * p.k.st), 0, valid, ks);
     vload.issue(reinterpret_cast<const char *>(vbase + (int64_t)key0 * p.v.st), 0, valid, ks + TL::kBytes);
   };
@@ -722,7 +730,7 @@ size_t mfma_fwd_workspace_bytes(const FwdParams &p) {
 bool mfma_fwd_supported(const FwdParams &p, int dtype) {
   return (dtype == DK_BF16 || dtype == DK_F16) && mfma_head_dim_ok(p.D) && p.csr.block_rows == 64 &&
          p.csr.block_cols == 64 && p.vec_ok &&
-         (p.csr.entry_width == 1 || p.csr.sub_block != 0) &&
+         (p.csr.entry_width == 1 || p.csr.sub_block != 0) && mfma_row_bytes_ok(p.k) && mfma_row_bytes_ok(p.v) &&
          p.scale_log2 > 0.f;  // the row maximum is taken before scaling (a scale <= 0 runs on the generic kernels)
 }
 

@@ -46,6 +46,24 @@ def test_out_kwarg_unpadded(impl):
     assert torch.isnan(big[:, :5]).all() and torch.isnan(big[:, :, Hq]).all()   # nothing else was written
 
 
+@pytest.mark.parametrize("D", [64, 128])
+def test_out_rows_not_cache_line_aligned(D):
+    """Output rows that start 16 bytes into a 128-byte line and are 16 bytes longer than the
+    head dim apart: the whole-row stores must write exactly the rows' bytes."""
+    B, Hq, Hkv, L = 1, 4, 2, 200
+    sm = 1 / math.sqrt(D)
+    q, k, v = make_qkv(B, L, L, Hq, Hkv, D, torch.bfloat16)
+    big = torch.full((B, L, Hq, D + 8), float("nan"), dtype=torch.bfloat16, device=DEV)
+    out = big[..., 8:]
+    assert out.data_ptr() % 128 == 16 and (out.stride(2) * 2) % 128 != 0
+    mod = New(Hq, 256, 64, 2, 3, num_kv_heads=Hkv, out=out).to(DEV)
+    res = mod(q.to(DEV), k.to(DEV), v.to(DEV), sm)
+    assert res.data_ptr() == out.data_ptr()
+    ro, _ = oracle_fwd(q, k, v, _bm(Hq, 256, 2, 3, Hkv), 64, sm)
+    assert_close("O", out, ro, **TOL)
+    assert torch.isnan(big[..., :8]).all()   # the gaps between the rows were not written
+
+
 def test_out_kwarg_is_checked():
     q = torch.zeros(1, 128, 2, 64, dtype=torch.bfloat16, device=DEV)
     with pytest.raises(AssertionError, match="out has shape"):

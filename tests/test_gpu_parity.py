@@ -172,6 +172,23 @@ def test_seq_dim_and_non_contiguous(impl):
     run_fwd_bwd(2, 4, 4, 512, 128, torch.bfloat16, 64, seq_dim=2, non_contiguous=True)
 
 
+def test_keys_broadcast_along_tokens(impl):
+    """K and V expanded along the token dim (token stride 0, below the head dim): the tile
+    copies of the matrix-core kernels do not take such rows, the call must still be exact."""
+    B, H, L, D = 1, 2, 256, 128
+    sm_scale = 1.0 / math.sqrt(D)
+    q, k, v = make_qkv(B, L, L, H, H, D, torch.bfloat16)
+    k1, v1 = k[:, :1], v[:, :1]
+    mod = _module(H, L, 64, 2, 2)
+    ref_o, ref_lse = oracle_fwd(q.float(), k1.expand(-1, L, -1, -1).float(), v1.expand(-1, L, -1, -1).float(),
+                                _block_mask(H, L, 64, 2, 2), 64, sm_scale)
+    kd, vd = k1.to(DEV).expand(-1, L, -1, -1), v1.to(DEV).expand(-1, L, -1, -1)
+    assert kd.stride(1) == 0
+    out, lse = mod(q.to(DEV), kd, vd, sm_scale, return_lse=True)
+    assert_close("O", out, ref_o, **TOL)
+    assert_close("LSE", lse, ref_lse, atol=LSE_TOL, rtol=0)
+
+
 def test_noncausal(impl):
     run_fwd_bwd(1, 2, 2, 1024, 64, torch.float16, 64, 4, 8, causal=False)
     run_fwd_bwd(1, 1, 1, 1024, 64, torch.float16, 32, 4, 10000, causal=False)

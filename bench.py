@@ -158,7 +158,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the path has no cross-GPU component in this build "
-              "(heads and KV partitions shard without communication; see DESIGN.md). Use --gpus 1.",
+              "(heads and KV partitions shard without communication). Use --gpus 1.",
               file=sys.stderr)
         sys.exit(2)
 

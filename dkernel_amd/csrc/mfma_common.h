@@ -101,6 +101,29 @@ __device__ __forceinline__ V lds_read8(const char *p) {
   return as_vec8<V>(*reinterpret_cast<const uint4 *>(p));
 }
 
+// The same reads from 32-bit LDS byte addresses.  Loop-invariant per-lane addresses are kept as
+// such integers and passed through opaque_lds_address once: left as pointer arithmetic the
+// compiler splits them into a row part and a chunk part and adds the two again in front of
+// every read (8 + 16 additions per 64 x 64 block in the forward).
+__device__ __forceinline__ uint32_t opaque_lds_address(uint32_t a) {
+  asm volatile("" : "+v"(a));
+  return a;
+}
+template <typename V>
+__device__ __forceinline__ V lds_read8_at(uint32_t addr) {
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  typedef const u32x4 __attribute__((address_space(3))) * lds_ptr;
+  return __builtin_bit_cast(V, *(lds_ptr)(uintptr_t)addr);
+}
+template <typename V>
+__device__ __forceinline__ V lds_read_tr8_at(uint32_t a0, uint32_t a1) {
+  typedef shortx4 __attribute__((address_space(3))) * lds_ptr;
+  shortx4 a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(uintptr_t)a0);
+  shortx4 b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(uintptr_t)a1);
+  shortx8 r = __builtin_shufflevector(a, b, 0, 1, 2, 3, 4, 5, 6, 7);
+  return __builtin_bit_cast(V, r);
+}
+
 // Two transpose reads -> the 8 k-values of one operand lane.
 template <typename V>
 __device__ __forceinline__ V lds_read_tr8(const char *p0, const char *p1) {
@@ -376,6 +399,29 @@ __device__ __forceinline__ void wait_tiles_ahead(int ahead) {
 }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// Maxima without the quieting step.  For fmaxf the compiler first passes every operand that
+// might be a signalling NaN through v_max_f32 x, x: 32 extra instructions for the 32 scores of
+// a softmax row share, more than the reduction itself.  The matrix unit does not produce
+// signalling NaNs, so the instructions are used directly.
+__device__ __forceinline__ float max2(float a, float b) {
+  float d;
+  asm("v_max_f32 %0, %1, %2" : "=v"(d) : "v"(a), "v"(b));
+  return d;
+}
+__device__ __forceinline__ float max3(float a, float b, float c) {
+  float d;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "v"(b), "v"(c));
+  return d;
+}
+// Maximum of a lane's value and the one of the lane 32 away (one VALU exchange, no LDS round
+// trip: v_permlane32_swap of (x, x) leaves the lower half's values in one result and the upper
+// half's in the other).
+__device__ __forceinline__ float max_with_other_half(float x) {
+  const unsigned u = __builtin_bit_cast(unsigned, x);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return max2(__builtin_bit_cast(float, r[0]), __builtin_bit_cast(float, r[1]));
+}
 
 // Exchange with the lane 32 away (the other half-wave that holds the rest of
 // an accumulator row).

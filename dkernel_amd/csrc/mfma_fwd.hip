@@ -162,14 +162,16 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
   // chunk 2ks+g; transpose-read pairs of d-tile dt); tile / k-step row offsets are immediates
   // (full pointers, and the stage is a compile-time constant of the loop body, so that stage,
   // tile and k-step offsets all end up as instruction immediates)
-  const char *rd[KS], *tr[DT][2];
+  uint32_t rd[KS], tr[DT][2];
   {
     int tro[DT][2];
     transposed_offsets<D>(lane, tro);
+    const uint32_t smem_lds = lds_address(smem);
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) rd[ks] = smem + TL::off(m, 2 * ks + g);
+    for (int ks = 0; ks < KS; ++ks) rd[ks] = opaque_lds_address(smem_lds + TL::off(m, 2 * ks + g));
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) tr[dt][0] = smem + tro[dt][0], tr[dt][1] = smem + tro[dt][1];
+    for (int dt = 0; dt < DT; ++dt)
+      tr[dt][0] = opaque_lds_address(smem_lds + tro[dt][0]), tr[dt][1] = opaque_lds_address(smem_lds + tro[dt][1]);
   }
 
   // Table entries: block e in col_cur (scalar register); block e + 1 is requested one block
@@ -259,26 +261,26 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
         for (int kb = 0; kb < KS; kb += 8) {
           vec8 ka[8];
 #pragma unroll
-          for (int i = 0; i < 8; ++i) ka[i] = lds_read8<vec8>(rd[kb + i] + ks_ + nt * 32 * TL::kRowBytes);
+          for (int i = 0; i < 8; ++i) ka[i] = lds_read8_at<vec8>(rd[kb + i] + ks_ + nt * 32 * TL::kRowBytes);
           __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
           for (int i = 0; i < 8; ++i) sacc[nt] = M::mma(ka[i], qf[kb + i], sacc[nt]);
           __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) va[0][dt] = lds_read_tr8<vec8>(tr[dt][0] + vs_, tr[dt][1] + vs_);
+      for (int dt = 0; dt < DT; ++dt) va[0][dt] = lds_read_tr8_at<vec8>(tr[dt][0] + vs_, tr[dt][1] + vs_);
     } else {
       vec8 ka[2][KS];
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) ka[0][ks] = lds_read8<vec8>(rd[ks] + ks_);
+      for (int ks = 0; ks < KS; ++ks) ka[0][ks] = lds_read8_at<vec8>(rd[ks] + ks_);
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) ka[1][ks] = lds_read8<vec8>(rd[ks] + ks_ + 32 * TL::kRowBytes);
+      for (int ks = 0; ks < KS; ++ks) ka[1][ks] = lds_read8_at<vec8>(rd[ks] + ks_ + 32 * TL::kRowBytes);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) sacc[0] = M::mma(ka[0][ks], qf[ks], sacc[0]);
       // first V^T operands do not depend on the softmax: fetch them behind the multiplies
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) va[0][dt] = lds_read_tr8<vec8>(tr[dt][0] + vs_, tr[dt][1] + vs_);
+      for (int dt = 0; dt < DT; ++dt) va[0][dt] = lds_read_tr8_at<vec8>(tr[dt][0] + vs_, tr[dt][1] + vs_);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) sacc[1] = M::mma(ka[1][ks], qf[ks], sacc[1]);
@@ -317,10 +319,10 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
           sacc[nt][r] = key > lim ? -INFINITY : sacc[nt][r];
         }
     }
-    float mx = fmaxf(sacc[0][0], sacc[1][0]);
+    float mx = max2(sacc[0][0], sacc[1][0]);
 #pragma unroll
-    for (int r = 1; r < 16; ++r) mx = fmaxf(mx, fmaxf(sacc[0][r], sacc[1][r]));
-    mx = fmaxf(mx, xor32(mx)) * p.scale_log2;  // scale > 0: max commutes with it
+    for (int r = 1; r < 16; ++r) mx = max3(mx, sacc[0][r], sacc[1][r]);
+    mx = max_with_other_half(mx) * p.scale_log2;  // scale > 0: max commutes with it
     if (__builtin_amdgcn_ballot_w64(mx > m_run + 8.f) != 0) {  // wave-uniform: some row needs a new reference
       const float m_new = fmaxf(m_run, mx);
       const float alpha = fast_exp2(m_run - (m_new == -INFINITY ? 0.f : m_new));
@@ -356,7 +358,7 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
       if (step < 3) {
         const int vrow = vs_ + ((step + 1) * 16) * TL::kRowBytes;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) va[(step + 1) & 1][dt] = lds_read_tr8<vec8>(tr[dt][0] + vrow, tr[dt][1] + vrow);
+        for (int dt = 0; dt < DT; ++dt) va[(step + 1) & 1][dt] = lds_read_tr8_at<vec8>(tr[dt][0] + vrow, tr[dt][1] + vrow);
       }
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) oacc[dt] = M::mma(va[step & 1][dt], pb, oacc[dt]);
@@ -512,7 +514,7 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
   };
   // raise the reference maximum if some row's maximum grew by more than 2^8 (rare, wave-uniform)
   auto new_reference = [&](float mx) {
-    mx = fmaxf(mx, xor32_swap(mx)) * p.scale_log2;
+    mx = max_with_other_half(mx) * p.scale_log2;
     if (__builtin_amdgcn_ballot_w64(mx > m_run + 8.f) != 0) {
       const float m_new = fmaxf(m_run, mx);
       const float alpha = fast_exp2(m_run - (m_new == -INFINITY ? 0.f : m_new));
@@ -544,7 +546,7 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
 #pragma unroll
     for (int e = 0; e < 32; ++e) {
       sa[e >> 4][e & 15] = masked(sa[e >> 4][e & 15], e, lim);
-      mx = fmaxf(mx, sa[e >> 4][e & 15]);
+      mx = max2(mx, sa[e >> 4][e & 15]);
     }
     new_reference(mx);
   }
@@ -620,7 +622,7 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
 #pragma unroll
           for (int e = (step * DT + dt) * PERC; e < (step * DT + dt + 1) * PERC; ++e) {
             snext[e >> 4][e & 15] = masked(snext[e >> 4][e & 15], e, lim);
-            mx = fmaxf(mx, snext[e >> 4][e & 15]);
+            mx = max2(mx, snext[e >> 4][e & 15]);
           }
           __builtin_amdgcn_sched_barrier(0);
         }

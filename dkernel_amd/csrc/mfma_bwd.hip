@@ -326,19 +326,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 
   for (int i = 0; i < DT / 2; ++i) {
 #pragma unroll
     for (int r4 = 0; r4 < 4; ++r4) {
-      T o4[4];
+      float f4[4];
       const int dt = kh * (DT / 2) + i;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int r = r4 * 4 + j;
         const float own = kh == 0 ? acc[i][r] : acc[DT / 2 + i][r];
-        o4[j] = from_float<T>((own + red[((rh * DT + dt) * 16 + r) * 64 + lane]) * p.sm_scale);
+        f4[j] = (own + red[((rh * DT + dt) * 16 + r) * 64 + lane]) * p.sm_scale;
       }
+      const uint2 o4 = pack4<T>(f4[0], f4[1], f4[2], f4[3]);
       // registers 4*r4 .. 4*r4+3 are dims 32dt + 8r4 + 4g + {0..3}
       if constexpr (kStagedStores)
-        *reinterpret_cast<uint2 *>(out_tile + TL::off(rh * 32 + m_late, dt * 4 + r4) + g_late * 8) = *reinterpret_cast<const uint2 *>(o4);
+        *reinterpret_cast<uint2 *>(out_tile + TL::off(rh * 32 + m_late, dt * 4 + r4) + g_late * 8) = o4;
       else if (!PAD || dt * 32 + r4 * 8 + g * 4 < p.D)
-        *reinterpret_cast<uint2 *>(dqp + dt * 32 + r4 * 8 + g * 4) = *reinterpret_cast<const uint2 *>(o4);
+        *reinterpret_cast<uint2 *>(dqp + dt * 32 + r4 * 8 + g * 4) = o4;
     }
   }
   if constexpr (kStagedStores) {
@@ -737,11 +738,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
       for (int r4 = 0; r4 < 4; ++r4) {
-        T o4[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) o4[i] = from_float<T>(acc[dt][r4 * 4 + i] * out_scale);
         if (!PAD || dt * 32 + r4 * 8 + g * 4 < p.D)
-          *reinterpret_cast<uint2 *>(outp + dt * 32 + r4 * 8 + g * 4) = *reinterpret_cast<const uint2 *>(o4);
+          *reinterpret_cast<uint2 *>(outp + dt * 32 + r4 * 8 + g * 4) =
+              pack4<T>(acc[dt][r4 * 4] * out_scale, acc[dt][r4 * 4 + 1] * out_scale, acc[dt][r4 * 4 + 2] * out_scale,
+                       acc[dt][r4 * 4 + 3] * out_scale);
       }
   }
 }

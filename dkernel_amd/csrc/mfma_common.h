@@ -70,6 +70,18 @@ struct Mma<f16_t> {
   }
 };
 
+// Four floats to four 16-bit values (round to nearest even) with the hardware conversions
+// (v_cvt_pk_bf16_f32 / v_cvt_f16_f32), 8 bytes ready to store.  The generic `from_float` for
+// bf16 is integer arithmetic with a NaN branch, some ten instructions per value: at 64 values
+// per lane that was the larger part of the forward's close-down.
+template <typename T>
+__device__ __forceinline__ uint2 pack4(float a, float b, float c, float d) {
+  using E = typename Mma<T>::elem;
+  typedef E v4 __attribute__((ext_vector_type(4)));
+  const v4 r = {(E)a, (E)b, (E)c, (E)d};
+  return __builtin_bit_cast(uint2, r);
+}
+
 // acc + dot product of two 16-byte groups of eight 16-bit values (exact fp32 products)
 template <typename T>
 __device__ __forceinline__ float dot8(uint4 a, uint4 b, float acc);
@@ -364,10 +376,9 @@ __device__ __forceinline__ void store_tile_rows(char *stage, const floatx16 (&ac
 #pragma unroll
     for (int r4 = 0; r4 < 4; ++r4) {
       // registers 4*r4 .. 4*r4+3 are dims 32dt + 8r4 + 4g + {0..3}
-      T o4[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) o4[i] = from_float<T>(acc[dt][r4 * 4 + i] * row_scale);
-      *reinterpret_cast<uint2 *>(stage + TL::off(m, dt * 4 + r4) + g * 8) = *reinterpret_cast<const uint2 *>(o4);
+      *reinterpret_cast<uint2 *>(stage + TL::off(m, dt * 4 + r4) + g * 8) =
+          pack4<T>(acc[dt][r4 * 4] * row_scale, acc[dt][r4 * 4 + 1] * row_scale, acc[dt][r4 * 4 + 2] * row_scale,
+                   acc[dt][r4 * 4 + 3] * row_scale);
     }
   store_staged_rows<T, D, PAD, 32>(stage, g_row0, row_stride, lane, row_lo, row_hi, real_d);
 }

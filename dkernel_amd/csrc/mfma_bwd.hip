@@ -132,7 +132,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 
   auto issue = [&](int col, int stage) {  // asynchronous copy of K/V block `col` into `stage`
     const int key0 = col * 64;
     char *ks = smem + stage * STAGE;
-    if ((uint32_t)key0 < k_full_span) {  // main path (one scalar compare; a padding entry is negative)
+    // (not at the 256-wide tile: the extra scalar state pushes those kernels into scratch spills)
+    if (D <= 128 && (uint32_t)key0 < k_full_span) {  // main path (one scalar compare; a padding entry is negative)
       kload.issue_full(row_address(reinterpret_cast<const char *>(kbase), key0, k_row_bytes), ks);
       vload.issue_full(row_address(reinterpret_cast<const char *>(vbase), key0, v_row_bytes), ks + TL::kBytes);
       return;
@@ -144,15 +145,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 
   // operand read addresses inside this wave's key half (row kh*32 + m, chunk 2ks+g swizzled;
   // transpose-read pairs) for a tile at offset 0: full pointers, and the stage is a compile-time
   // constant of the loop body, so that stage and k-step offsets are instruction immediates
-  const char *rd[KS], *tr[DT][2];
+  using OA = OperandAddress<D>;
+  typename OA::type rd[KS], tr[DT][2];
   {
     int tro[DT][2];
     transposed_offsets<D>(lane, tro);
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) rd[ks] = smem + TL::off(kh * 32 + m, 2 * ks + g);
+    for (int ks = 0; ks < KS; ++ks) rd[ks] = OA::make(smem, TL::off(kh * 32 + m, 2 * ks + g));
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-      tr[dt][0] = smem + kh * 32 * TL::kRowBytes + tro[dt][0], tr[dt][1] = smem + kh * 32 * TL::kRowBytes + tro[dt][1];
+    for (int dt = 0; dt < DT; ++dt) {
+      tr[dt][0] = OA::make(smem, kh * 32 * TL::kRowBytes + tro[dt][0]);
+      tr[dt][1] = OA::make(smem, kh * 32 * TL::kRowBytes + tro[dt][1]);
+    }
   }
 
   floatx16 acc[DT];
@@ -227,7 +231,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 
     for (int half = 0; half < 2; ++half) {
       vec8 ka[KS / 2];
 #pragma unroll
-      for (int i = 0; i < KS / 2; ++i) ka[i] = lds_read8<vec8>(rd[half * (KS / 2) + i] + ks_);
+      for (int i = 0; i < KS / 2; ++i) ka[i] = lds_operand<vec8>(rd[half * (KS / 2) + i] + ks_);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < KS / 2; ++i) s = M::mma(ka[i], qf[half * (KS / 2) + i], s);
@@ -236,7 +240,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 
     for (int half = 0; half < 2; ++half) {
       vec8 va[KS / 2];
 #pragma unroll
-      for (int i = 0; i < KS / 2; ++i) va[i] = lds_read8<vec8>(rd[half * (KS / 2) + i] + vs_);
+      for (int i = 0; i < KS / 2; ++i) va[i] = lds_operand<vec8>(rd[half * (KS / 2) + i] + vs_);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < KS / 2; ++i) dp = M::mma(va[i], dof[half * (KS / 2) + i], dp);
@@ -244,7 +248,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 
     // K^T operands of the dQ product do not depend on dS: fetch them now
     vec8 kt[DT];
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) kt[dt] = lds_read_tr8<vec8>(tr[dt][0] + ks_, tr[dt][1] + ks_);
+    for (int dt = 0; dt < DT; ++dt) kt[dt] = lds_operand_tr<vec8>(tr[dt][0] + ks_, tr[dt][1] + ks_);
 
     const bool need_mask = (key0 + 31 >= sq.k_len) || (p.causal && key0 + 31 > row0);
     const int lim = p.causal ? min(pos, sq.k_len - 1) : sq.k_len - 1;  // last visible key of this row
@@ -283,7 +287,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 
       for (int dt = 0; dt < DT; ++dt) {
         acc[dt] = M::mma(kt[dt], dsb, acc[dt]);
         if (t == 0)  // refill with the second k-step's operand as soon as the register is free
-          kt[dt] = lds_read_tr8<vec8>(tr[dt][0] + ks_ + 16 * TL::kRowBytes, tr[dt][1] + ks_ + 16 * TL::kRowBytes);
+          kt[dt] = lds_operand_tr<vec8>(tr[dt][0] + ks_ + 16 * TL::kRowBytes, tr[dt][1] + ks_ + 16 * TL::kRowBytes);
       }
     }
   };
@@ -494,7 +498,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 
       char *dst = smem + S::kVec + qstage * 256;
       // main path: a listed block whose 32 rows all are queries (one scalar compare: a padding
       // entry, rbq < 0, gives a negative qi0)
-      if ((uint32_t)qi0 < full_span) {
+      if (D <= 128 && (uint32_t)qi0 < full_span) {
         qload.issue_full(row_address(reinterpret_cast<const char *>(qbase), qi0, q_row_bytes),
                          smem + S::kQ + qstage * S::kTile);
         doload.issue_full(row_address(reinterpret_cast<const char *>(dobase), qi0, do_row_bytes),

@@ -14,6 +14,7 @@
 // the transposed matrix, without ever storing the transpose.
 #pragma once
 
+#include <type_traits>
 #include <hip/hip_runtime.h>
 
 #include "device_common.h"
@@ -136,6 +137,23 @@ __device__ __forceinline__ V lds_read_tr8_at(uint32_t a0, uint32_t a1) {
   return __builtin_bit_cast(V, r);
 }
 
+__device__ __forceinline__ uint32_t lds_address(const void *p);  // below
+
+// Loop-invariant operand addresses of a kernel with D-wide tiles: opaque 32-bit LDS addresses
+// up to the 128-wide tile; at the 256-wide tile (32 addresses next to 128 accumulator
+// registers) plain pointers, which the compiler may rebuild instead of keeping them live.
+template <int D>
+struct OperandAddress {
+  static constexpr bool kOpaque = D <= 128;
+  using type = typename std::conditional<kOpaque, uint32_t, const char *>::type;
+  static __device__ __forceinline__ type make(char *smem, int offset) {
+    if constexpr (kOpaque)
+      return opaque_lds_address(lds_address(smem) + offset);
+    else
+      return smem + offset;
+  }
+};
+
 // Two transpose reads -> the 8 k-values of one operand lane.
 template <typename V>
 __device__ __forceinline__ V lds_read_tr8(const char *p0, const char *p1) {
@@ -145,6 +163,16 @@ __device__ __forceinline__ V lds_read_tr8(const char *p0, const char *p1) {
   shortx8 r = __builtin_shufflevector(a, b, 0, 1, 2, 3, 4, 5, 6, 7);
   return __builtin_bit_cast(V, r);
 }
+
+// Either kind of address (OperandAddress<D>::type)
+template <typename V>
+__device__ __forceinline__ V lds_operand(const char *p) { return lds_read8<V>(p); }
+template <typename V>
+__device__ __forceinline__ V lds_operand(uint32_t a) { return lds_read8_at<V>(a); }
+template <typename V>
+__device__ __forceinline__ V lds_operand_tr(const char *p0, const char *p1) { return lds_read_tr8<V>(p0, p1); }
+template <typename V>
+__device__ __forceinline__ V lds_operand_tr(uint32_t a0, uint32_t a1) { return lds_read_tr8_at<V>(a0, a1); }
 
 // ---------------------------------------------------------------------------
 // 64-row x D tile of 16-bit elements in LDS, row-major, with an XOR swizzle of

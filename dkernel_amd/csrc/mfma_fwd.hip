@@ -141,7 +141,9 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
   auto issue = [&](int col, int stage) {
     const int key0 = col * 64;
     char *ks = smem + stage * S::kStage;
-    if ((uint32_t)key0 < k_full_span) {  // main path (one scalar compare; a padding entry is negative)
+    // (not at the 256-wide tile, nor for one padded head per workgroup: the extra state pushes
+    // those instantiations into scratch spills)
+    if (D <= 128 && !(PAD && G == 1) && (uint32_t)key0 < k_full_span) {  // main path (one scalar compare; a padding entry is negative)
       kload.issue_full(row_address(reinterpret_cast<const char *>(kbase), key0, k_row_bytes), ks);
       vload.issue_full(row_address(reinterpret_cast<const char *>(vbase), key0, v_row_bytes), ks + TL::kBytes);
       return;
@@ -162,16 +164,15 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
   // chunk 2ks+g; transpose-read pairs of d-tile dt); tile / k-step row offsets are immediates
   // (full pointers, and the stage is a compile-time constant of the loop body, so that stage,
   // tile and k-step offsets all end up as instruction immediates)
-  uint32_t rd[KS], tr[DT][2];
+  using OA = OperandAddress<D>;
+  typename OA::type rd[KS], tr[DT][2];
   {
     int tro[DT][2];
     transposed_offsets<D>(lane, tro);
-    const uint32_t smem_lds = lds_address(smem);
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) rd[ks] = opaque_lds_address(smem_lds + TL::off(m, 2 * ks + g));
+    for (int ks = 0; ks < KS; ++ks) rd[ks] = OA::make(smem, TL::off(m, 2 * ks + g));
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-      tr[dt][0] = opaque_lds_address(smem_lds + tro[dt][0]), tr[dt][1] = opaque_lds_address(smem_lds + tro[dt][1]);
+    for (int dt = 0; dt < DT; ++dt) tr[dt][0] = OA::make(smem, tro[dt][0]), tr[dt][1] = OA::make(smem, tro[dt][1]);
   }
 
   // Table entries: block e in col_cur (scalar register); block e + 1 is requested one block
@@ -261,26 +262,26 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
         for (int kb = 0; kb < KS; kb += 8) {
           vec8 ka[8];
 #pragma unroll
-          for (int i = 0; i < 8; ++i) ka[i] = lds_read8_at<vec8>(rd[kb + i] + ks_ + nt * 32 * TL::kRowBytes);
+          for (int i = 0; i < 8; ++i) ka[i] = lds_operand<vec8>(rd[kb + i] + ks_ + nt * 32 * TL::kRowBytes);
           __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
           for (int i = 0; i < 8; ++i) sacc[nt] = M::mma(ka[i], qf[kb + i], sacc[nt]);
           __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) va[0][dt] = lds_read_tr8_at<vec8>(tr[dt][0] + vs_, tr[dt][1] + vs_);
+      for (int dt = 0; dt < DT; ++dt) va[0][dt] = lds_operand_tr<vec8>(tr[dt][0] + vs_, tr[dt][1] + vs_);
     } else {
       vec8 ka[2][KS];
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) ka[0][ks] = lds_read8_at<vec8>(rd[ks] + ks_);
+      for (int ks = 0; ks < KS; ++ks) ka[0][ks] = lds_operand<vec8>(rd[ks] + ks_);
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) ka[1][ks] = lds_read8_at<vec8>(rd[ks] + ks_ + 32 * TL::kRowBytes);
+      for (int ks = 0; ks < KS; ++ks) ka[1][ks] = lds_operand<vec8>(rd[ks] + ks_ + 32 * TL::kRowBytes);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) sacc[0] = M::mma(ka[0][ks], qf[ks], sacc[0]);
       // first V^T operands do not depend on the softmax: fetch them behind the multiplies
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) va[0][dt] = lds_read_tr8_at<vec8>(tr[dt][0] + vs_, tr[dt][1] + vs_);
+      for (int dt = 0; dt < DT; ++dt) va[0][dt] = lds_operand_tr<vec8>(tr[dt][0] + vs_, tr[dt][1] + vs_);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) sacc[1] = M::mma(ka[1][ks], qf[ks], sacc[1]);
@@ -358,7 +359,7 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
       if (step < 3) {
         const int vrow = vs_ + ((step + 1) * 16) * TL::kRowBytes;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) va[(step + 1) & 1][dt] = lds_read_tr8_at<vec8>(tr[dt][0] + vrow, tr[dt][1] + vrow);
+        for (int dt = 0; dt < DT; ++dt) va[(step + 1) & 1][dt] = lds_operand_tr<vec8>(tr[dt][0] + vrow, tr[dt][1] + vrow);
       }
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) oacc[dt] = M::mma(va[step & 1][dt], pb, oacc[dt]);

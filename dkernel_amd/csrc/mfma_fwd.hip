@@ -58,7 +58,8 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
   constexpr int EW = SUB ? 2 : 1;  // ints per table entry
   SeqInfo sq;
   int tile;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: row tests and head indices follow it
   int rb;
   int first_rb = 0, last_rb = 0;  // RP: table rows that hold queries of this sequence
   if constexpr (RP) {

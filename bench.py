@@ -31,8 +31,8 @@ HBM_PEAK_GBS = 8000.0            # MI355X HBM3E, vendor figure
 # calibration + WRITE_SIZE; profiles/fwd_bwd_decode_counters.md).  Counters cannot be read from
 # inside this process, so these are quoted, not measured live.
 TRAFFIC_BYTES = {
-    "fwd": 222.4e6 + 136.3e6,
-    "bwd": (612.3e6 + 68.2e6) + (567.7e6 + 134.2e6),   # dQ pass + dK/dV pass
+    "fwd": 220.9e6 + 136.3e6,
+    "bwd": (611.9e6 + 68.2e6) + (570.1e6 + 134.2e6),   # dQ pass + dK/dV pass
     "decode": 180.5e6 + 0.3e6,
 }
 BS, LOCAL, VERT, D = 64, 16, 8, 128

@@ -173,8 +173,8 @@ def test_seq_dim_and_non_contiguous(impl):
 
 
 def test_keys_broadcast_along_tokens(impl):
-    """K and V expanded along the token dim (token stride 0, below the head dim): the tile
-    copies of the matrix-core kernels do not take such rows, the call must still be exact."""
+    """K and V expanded along the token dim (token stride 0): every row of a K/V tile is the
+    same memory, which the tile copies' 32-bit row offsets must handle like any other stride."""
     B, H, L, D = 1, 2, 256, 128
     sm_scale = 1.0 / math.sqrt(D)
     q, k, v = make_qkv(B, L, L, H, H, D, torch.bfloat16)

@@ -27,7 +27,6 @@
 // CU (2 per SIMD, <= 256 VGPRs each): one wave's loads overlap the other's
 // multiplies on the same SIMD.
 #include <algorithm>
-#include <cstdlib>
 #include <type_traits>
 
 #include "common.h"
@@ -48,10 +47,8 @@ static int decode_max_row_entries(const FwdParams &p) {
 // machine, a row is cut into as many units as a workgroup has waves, so that it is finished
 // inside one workgroup and the merge kernel is not launched at all; with few rows, into more
 // units (about 1024 waves in total).  At most 16 (the paged path keeps a unit's page numbers in
-// the lanes of one register).  DKERNEL_DECODE_UNIT overrides.
+// the lanes of one register).
 static int decode_unit_blocks(const FwdParams &p) {
-  static const int forced = getenv("DKERNEL_DECODE_UNIT") ? atoi(getenv("DKERNEL_DECODE_UNIT")) : 0;  // read once
-  if (forced >= 1 && forced <= 16) return forced;
   const int rows = p.seqs.batch * p.Hkv;
   const int units_per_row = std::max(kDecodeWaves, cdiv(1024, rows > 0 ? rows : 1));
   return std::min(16, std::max(2, cdiv(decode_max_row_entries(p), units_per_row)));
@@ -136,8 +133,8 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(2, 2))) 
   // never more than the host sized the grid and the workspace for: a row longer than the caller's
   // max_row_entries hint said is still cut into max_units units, each with a larger share
   const int u_cnt = min(decode_row_units(n_ent, unit_blocks, W), max_units);
-  if ((int)blockIdx.x * W >= u_cnt && (blockIdx.x > 0 || W == 1)) return;  // nothing for this workgroup
-  const bool merge_here = W > 1 && u_cnt <= W;  // (a row without entries is written here too: O = 0, LSE = -inf)
+  if ((int)blockIdx.x * W >= u_cnt && blockIdx.x > 0) return;  // nothing for this workgroup
+  const bool merge_here = u_cnt <= W;  // (a row without entries is written here too: O = 0, LSE = -inf)
   const int per = u_cnt > 0 ? (n_ent + u_cnt - 1) / u_cnt : 0;
   const int unit = blockIdx.x * W + wave;
   const bool active = unit < u_cnt;
@@ -395,7 +392,7 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(2, 2))) 
       dst[D + 1] = l_run;
     }
   }
-  if constexpr (W > 1) {
+  {
     if (!merge_here) return;
     __syncthreads();  // every wave of the workgroup gets here (merge_here is workgroup-uniform)
     // heads of the group are dealt to the waves; lane l owns dims l D/64 .. of its head
@@ -453,10 +450,10 @@ __global__ __launch_bounds__(64) void decode_combine_kernel(const FwdParams p, c
   if (sq.k_len > 0 && rb < p.csr.num_rows) {
     const int lh = lut_head(p.csr, h, p.Hq, p.Hkv);
     const int n = scalar_load(p.csr.ptr + lh * p.csr.ptr_sh + rb + 1) - scalar_load(p.csr.ptr + lh * p.csr.ptr_sh + rb);
-    units = min(decode_row_units(n, unit_blocks, merged_units > 0 ? merged_units : 1), max_units);  // as the partial kernel
+    units = min(decode_row_units(n, unit_blocks, merged_units), max_units);  // as the partial kernel
   }
-  // rows of at most merged_units units were finished by the partial kernel (merged_units > 0)
-  if (merged_units > 0 && units <= merged_units) return;
+  // rows of at most merged_units units (the waves of a partial-kernel workgroup) were finished there
+  if (units <= merged_units) return;
   const float *src = ws + ((int64_t)b * p.Hq + h) * max_units * (D + 2);
   float mmax = -INFINITY, l = 0.f, o[PER];
 #pragma unroll
@@ -519,8 +516,9 @@ size_t decode_workspace_bytes(const FwdParams &p) {
   return (size_t)p.seqs.batch * p.Hq * decode_max_units(p) * (mfma_tile_width(p.D) + 2) * sizeof(float);
 }
 
-template <typename T, int D, bool PAD, bool SUB, bool PAGED, bool KV8, int W>
-static int launch_decode_tdw(const FwdParams &p, float *ws, hipStream_t stream) {
+template <typename T, int D, bool PAD, bool SUB, bool PAGED, bool KV8 = false>
+static int launch_decode_td(const FwdParams &p, float *ws, hipStream_t stream) {
+  constexpr int W = kDecodeWaves;
   const int smem = W * DecSmem<D>::wave_bytes(p.Hq / p.Hkv);
   const int unit_blocks = decode_unit_blocks(p), max_units = decode_max_units(p);
   const int groups = cdiv(max_units, W);
@@ -530,20 +528,11 @@ static int launch_decode_tdw(const FwdParams &p, float *ws, hipStream_t stream) 
   hipLaunchKernelGGL((decode_partial_kernel<T, D, PAD, SUB, PAGED, KV8, W>), dim3(groups, p.Hkv, p.seqs.batch),
                      dim3(64 * W), smem, stream, p, ws, unit_blocks, max_units);
   DK_HIP_CHECK(hipGetLastError());
-  if (W > 1 && groups == 1) return DK_OK;  // every row was finished inside its workgroup
+  if (groups == 1) return DK_OK;  // every row was finished inside its workgroup
   hipLaunchKernelGGL((decode_combine_kernel<T, D, PAD>), dim3(p.Hq, p.seqs.batch), dim3(64), 0, stream, p, ws,
-                     unit_blocks, max_units, W > 1 ? W : 0);
+                     unit_blocks, max_units, W);
   DK_HIP_CHECK(hipGetLastError());
   return DK_OK;
-}
-
-// DKERNEL_DECODE_WAVES=1: one unit per workgroup and every row merged by the second kernel
-// (A/B measurements); default: kDecodeWaves units per workgroup.
-template <typename T, int D, bool PAD, bool SUB, bool PAGED, bool KV8 = false>
-static int launch_decode_td(const FwdParams &p, float *ws, hipStream_t stream) {
-  static const bool single = getenv("DKERNEL_DECODE_WAVES") && atoi(getenv("DKERNEL_DECODE_WAVES")) == 1;
-  if (single) return launch_decode_tdw<T, D, PAD, SUB, PAGED, KV8, 1>(p, ws, stream);
-  return launch_decode_tdw<T, D, PAD, SUB, PAGED, KV8, kDecodeWaves>(p, ws, stream);
 }
 
 template <typename T, bool PAGED>

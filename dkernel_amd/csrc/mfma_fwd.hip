@@ -19,8 +19,6 @@
 // Grid: x = head group (fastest, so that the 8 XCDs, which receive
 // workgroups round-robin, each keep a fixed set of kv heads in their L2),
 // y = q tile with the longest rows first, z = batch.
-#include <cstdlib>
-
 #include "common.h"
 #include "device_common.h"
 #include "mfma_common.h"
@@ -398,269 +396,12 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
   }
 }
 
-// ---------------------------------------------------------------------------
-// Software-pipelined variant: the QK^T multiplies of block j+1 are issued
-// before the softmax of block j, so the matrix pipe works while the VALU does
-// the exponentials (two independent instruction streams inside one wave).
-// K tiles therefore run one block ahead of V tiles; both rings have two
-// stages.  Same work split, grid and results as mfma_fwd_kernel.  Used for
-// one head per workgroup (G = 1, one wave per SIMD), where it measures faster.
-// ---------------------------------------------------------------------------
-template <typename T, int D, int G, bool PAD>
-__global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 ? 1 : 2, 2))) void mfma_fwd_pipe_kernel(
-    const FwdParams p, int tiles_y) {
-  using M = Mma<T>;
-  using vec8 = typename M::vec8;
-  using TL = Tile<D>;
-  constexpr int NT = 128 * G;
-  constexpr int KS = D / 16;
-  constexpr int DT = D / 32;
-  extern __shared__ __align__(16) char smem[];  // K stage 0, K stage 1, V stage 0, V stage 1
-
-  SeqInfo sq;
-  int tile;
-  const int ty = tiles_y - 1 - (int)blockIdx.y;  // longest rows first
-  if (!resolve_tile(p.seqs, p.causal, 64, 1, ty, blockIdx.z, sq, tile)) return;
-  const int rb = sq.past / 64 + tile;
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  if constexpr (PAD) {  // the slots of the head dims beyond p.D stay zero for the whole kernel
-    zero_tiles<NT>(smem, 4 * TL::kBytes, tid);
-    __syncthreads();
-  }
-  const int h = blockIdx.x * G + (wave >> 1);
-  const int kvh = __builtin_amdgcn_readfirstlane(h / (p.Hq / p.Hkv));  // integer division runs on the VALU
-  const int m = lane & 31, g = lane >> 5;
-  const int row0 = rb * 64 + (wave & 1) * 32;
-  const int pos = row0 + m;
-  const int qi = pos - sq.past;
-  const bool row_ok = qi >= 0 && qi < sq.q_len;
-
-  vec8 qf[KS];
-  {
-    const T *qp = (const T *)p.q.ptr + sq.b * p.q.sb + h * p.q.sh + (int64_t)(sq.q_start + qi) * p.q.st;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      uint4 w = make_uint4(0, 0, 0, 0);
-      if (row_ok && (!PAD || ks * 16 + g * 8 < p.D)) w = *reinterpret_cast<const uint4 *>(qp + ks * 16 + g * 8);
-      qf[ks] = as_vec8<vec8>(w);
-    }
-  }
-  const int lh = lut_head(p.csr, blockIdx.x * G, p.Hq, p.Hkv);
-  int e0 = 0, e1 = 0;
-  if (rb < p.csr.num_rows)
-    scalar_load2(p.csr.ptr + lh * p.csr.ptr_sh + rb, p.csr.ptr + lh * p.csr.ptr_sh + rb + 1, e0, e1);
-  const int n = e1 - e0;
-  const int32_t *cols = p.csr.idx + lh * p.csr.idx_sh + e0;
-  const T *kbase = (const T *)p.k.ptr + sq.b * p.k.sb + kvh * p.k.sh + (int64_t)sq.k_start * p.k.st;
-  const T *vbase = (const T *)p.v.ptr + sq.b * p.v.sb + kvh * p.v.sh + (int64_t)sq.k_start * p.v.st;
-
-  TileLoader<D, NT, PAD> kload, vload;
-  kload.init(tid, p.k.st, p.D);
-  vload.init(tid, p.v.st, p.D);
-  // table entries are read well before they are needed and never between a tile request and
-  // its wait (a vector load there would make the wait cover the tile just requested)
-  auto col_at = [&](int j) { return __builtin_amdgcn_readfirstlane(j < n ? cols[j] : 0); };
-  auto issue_k = [&](int stage, int col) {
-    const int key0 = col * 64;
-    kload.issue(reinterpret_cast<const char *>(kbase + (int64_t)key0 * p.k.st), 0, col < 0 ? 0 : sq.k_len - key0,
-                smem + stage * TL::kBytes);
-  };
-  auto issue_v = [&](int stage, int col) {
-    const int key0 = col * 64;
-    vload.issue(reinterpret_cast<const char *>(vbase + (int64_t)key0 * p.v.st), 0, col < 0 ? 0 : sq.k_len - key0,
-                smem + (2 + stage) * TL::kBytes);
-  };
-  // loop-invariant LDS addresses of this lane's operand reads inside a tile at offset 0 (full
-  // pointers, so that stage, tile and k-step offsets are instruction immediates)
-  const char *rd[KS], *tr[DT][2];
-  {
-    int tro[DT][2];
-    transposed_offsets<D>(lane, tro);
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) rd[ks] = smem + TL::off(m, 2 * ks + g);
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt) tr[dt][0] = smem + tro[dt][0], tr[dt][1] = smem + tro[dt][1];
-  }
-
-  floatx16 oacc[DT];
-#pragma unroll
-  for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) oacc[dt][r] = 0.f;
-  float m_run = -INFINITY, l_run = 0.f;
-  floatx16 sa[2], sb[2];
-
-  // Every multiply is followed by a slice of this wave's own VALU work and a
-  // scheduler barrier, so that the VALU work is issued in the shadow of the
-  // multiply (a wave issues in order; with one wave per SIMD nothing else
-  // fills the matrix pipe while that wave does its exponentials).
-  //
-  // Slot s (0 .. 2KS-1) of S^T = K Q^T: 32-key tile s / KS, k-step s % KS.
-  constexpr int RING = 4;
-  auto k_operand = [&](int stage_off, int s) {
-    return lds_read8<vec8>(rd[s % KS] + stage_off + (s / KS) * 32 * TL::kRowBytes);
-  };
-  // mask of block `col` applied to S (wave-uniform decision)
-  auto block_needs_mask = [&](int col) {
-    const int key0 = col * 64;
-    return col < 0 || (key0 + 63 >= sq.k_len) || (p.causal && key0 + 63 > row0);
-  };
-  // last visible key of this row minus the block's first key (keys of the block are 0..63)
-  auto block_limit = [&](int col) {
-    return col < 0 ? -1 : (p.causal ? min(pos, sq.k_len - 1) : sq.k_len - 1) - col * 64;
-  };
-  auto masked = [&](float x, int e, int lim) {  // element e = 16 nt + r of the accumulator pair
-    const int key = (e >> 4) * 32 + ((e & 15) >> 2) * 8 + g * 4 + (e & 3);
-    return key > lim ? -INFINITY : x;
-  };
-  // raise the reference maximum if some row's maximum grew by more than 2^8 (rare, wave-uniform)
-  auto new_reference = [&](float mx) {
-    mx = max_with_other_half(mx) * p.scale_log2;
-    if (__builtin_amdgcn_ballot_w64(mx > m_run + 8.f) != 0) {
-      const float m_new = fmaxf(m_run, mx);
-      const float alpha = fast_exp2(m_run - (m_new == -INFINITY ? 0.f : m_new));
-      l_run *= alpha;
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
-      m_run = m_new;
-    }
-  };
-
-  int col_cur = col_at(0), col_next = col_at(1);  // blocks j and j+1 of the coming step
-  if (n > 0) {
-    issue_k(0, col_cur);
-    wait_tile_loads();
-    __syncthreads();
-    if (n > 1) issue_k(1, col_next);
-    issue_v(0, col_cur);
-    // S_0, its mask and row maximum: plain code, once per tile
-#pragma unroll
-    for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) sa[nt][r] = 0.f;
-#pragma unroll
-    for (int s_ = 0; s_ < 2 * KS; ++s_) sa[s_ / KS] = M::mma(k_operand(0, s_), qf[s_ % KS], sa[s_ / KS]);
-    const int lim = block_needs_mask(col_cur) ? block_limit(col_cur) : 64;
-    float mx = -INFINITY;
-#pragma unroll
-    for (int e = 0; e < 32; ++e) {
-      sa[e >> 4][e & 15] = masked(sa[e >> 4][e & 15], e, lim);
-      mx = max2(mx, sa[e >> 4][e & 15]);
-    }
-    new_reference(mx);
-  }
-  // one block: consumes S_j (scur), produces S_{j+1} (snext); the caller alternates the two
-  // accumulator pairs so that no copy is needed
-  auto block_step = [&](auto parity, int j, floatx16(&scur)[2], floatx16(&snext)[2]) {
-    constexpr int PAR = decltype(parity)::value;  // j & 1, a constant so that every LDS address is lane offset + immediate
-    const int col_next2 = col_at(j + 2);
-    wait_tile_loads();
-    __syncthreads();  // K_{j+1} and V_j are visible; every wave is done with K_j and V_{j-1}
-    if (j + 2 < n) issue_k(PAR, col_next2);
-    if (j + 1 < n) issue_v(PAR ^ 1, col_next);
-    constexpr int kn = (PAR ^ 1) * TL::kBytes;  // K_{j+1}
-    constexpr int vs_ = (2 + PAR) * TL::kBytes;  // V_j
-    const float m_use = m_run == -INFINITY ? 0.f : m_run;
-    // everything with a branch comes first: the two phases below must share one basic block,
-    // or the compiler sinks the exponentials out of the multiply loop
-    const bool more = j + 1 < n;
-    const int coln = col_next;
-    // masking is unconditional (limit 64 = nothing masked): two variants of the second phase
-    // in a branch cost more registers than the compare/select pairs cost issue slots there
-    const int lim = more && block_needs_mask(coln) ? block_limit(coln) : 64;
-
-    // ---- S_{j+1} = K_{j+1} Q^T (after the last block: of a stale tile, discarded)
-    //      in step with P_j = exp2(S_j scale - m)
-    vec8 pb[4];
-    float psum = 0.f;
-    {
-#pragma unroll
-      for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) snext[nt][r] = 0.f;
-      vec8 ka[RING];
-#pragma unroll
-      for (int s_ = 0; s_ < RING; ++s_) ka[s_] = k_operand(kn, s_);
-      constexpr int PER = 32 / (2 * KS);
-      static_assert(PER % 2 == 0, "probabilities are packed in pairs");
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int s_ = 0; s_ < 2 * KS; ++s_) {
-        snext[s_ / KS] = M::mma(ka[s_ % RING], qf[s_ % KS], snext[s_ / KS]);
-        if (s_ + RING < 2 * KS) ka[s_ % RING] = k_operand(kn, s_ + RING);
-#pragma unroll
-        for (int e = s_ * PER; e < (s_ + 1) * PER; ++e) {
-          const int step = e >> 3, idx = e & 7;
-          const float pv = fast_exp2(fmaf(scur[step >> 1][(step & 1) * 8 + idx], p.scale_log2, -m_use));
-          psum += pv;
-          pb[step][idx] = (typename M::elem)pv;
-        }
-        __builtin_amdgcn_sched_barrier(0);
-      }
-    }
-    l_run += psum;
-
-    // ---- O^T += V_j^T P_j^T in step with the mask and row maximum of S_{j+1}
-    float mx = -INFINITY;
-    {
-      vec8 va[DT];  // refilled for the next k-step right behind the multiply that consumed it
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt) va[dt] = lds_read_tr8<vec8>(tr[dt][0] + vs_, tr[dt][1] + vs_);
-      constexpr int PERC = 32 / (4 * DT);
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int step = 0; step < 4; ++step)
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-          oacc[dt] = M::mma(va[dt], pb[step], oacc[dt]);
-          if (step < 3) {
-            constexpr int vrow = vs_ + 16 * TL::kRowBytes;  // per k-step
-            va[dt] = lds_read_tr8<vec8>(tr[dt][0] + vrow * 1 + step * 16 * TL::kRowBytes,
-                                        tr[dt][1] + vrow * 1 + step * 16 * TL::kRowBytes);
-          }
-#pragma unroll
-          for (int e = (step * DT + dt) * PERC; e < (step * DT + dt + 1) * PERC; ++e) {
-            snext[e >> 4][e & 15] = masked(snext[e >> 4][e & 15], e, lim);
-            mx = max2(mx, snext[e >> 4][e & 15]);
-          }
-          __builtin_amdgcn_sched_barrier(0);
-        }
-    }
-    if (more) new_reference(mx);
-    col_next = col_next2;
-  };
-  for (int j = 0; j < n; j += 2) {
-    block_step(Const<0>{}, j, sa, sb);
-    if (j + 1 < n) block_step(Const<1>{}, j + 1, sb, sa);
-  }
-  l_run += xor32(l_run);
-
-  __syncthreads();  // the tile rings are free: each wave stages its O tile in 32 rows of them
-  const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
-  {
-    const int qi0 = row0 - sq.past;
-    T *o_row0 = (T *)p.o.ptr + sq.b * p.o.sb + h * p.o.sh + (int64_t)(sq.q_start + qi0) * p.o.st;
-    store_tile_rows<T, D, PAD>(smem + wave * 32 * TL::kRowBytes, oacc, inv, o_row0, p.o.st, lane, -qi0,
-                               sq.q_len - qi0, p.D);
-  }
-  if (!row_ok) return;
-  if (p.lse.ptr && g == 0) {
-    const float lse = l_run > 0.f ? (m_run + log2f(l_run)) * kLn2 : -INFINITY;
-    p.lse.ptr[sq.b * p.lse.sb + h * p.lse.sh + (int64_t)(sq.q_start + qi) * p.lse.st] = lse;
-  }
-}
-
 // Explicit instantiations: with only the implicit ones the fp16 host stubs of
 // this kernel are not emitted by this compiler version.
 #define DK_INSTANTIATE_FWD(T, D, PAD)                                                  \
-  template __global__ void mfma_fwd_kernel<T, D, 1, PAD, false>(const FwdParams, int); \
   template __global__ void mfma_fwd_kernel<T, D, 2, PAD, false>(const FwdParams, int); \
   template __global__ void mfma_fwd_kernel<T, D, 2, PAD, true>(const FwdParams, int);  \
-  template __global__ void mfma_fwd_kernel<T, D, 4, PAD, false>(const FwdParams, int); \
-  template __global__ void mfma_fwd_pipe_kernel<T, D, 1, PAD>(const FwdParams, int);
+  template __global__ void mfma_fwd_kernel<T, D, 4, PAD, false>(const FwdParams, int);
 #define DK_INSTANTIATE_FWD_SUB(T, D, PAD)                                                    \
   template __global__ void mfma_fwd_kernel<T, D, 1, PAD, false, true>(const FwdParams, int); \
   template __global__ void mfma_fwd_kernel<T, D, 2, PAD, false, true>(const FwdParams, int); \
@@ -676,7 +417,6 @@ DK_INSTANTIATE_FWD_SUB(f16_t, 64, true)
 #undef DK_INSTANTIATE_FWD_SUB
 // 256-wide tiles: the zero-padding instantiation only (it also takes head_dim 256 itself)
 #define DK_INSTANTIATE_FWD_256(T)                                                            \
-  template __global__ void mfma_fwd_kernel<T, 256, 1, true, false, false>(const FwdParams, int); \
   template __global__ void mfma_fwd_kernel<T, 256, 2, true, false, false>(const FwdParams, int); \
   template __global__ void mfma_fwd_kernel<T, 256, 2, true, true, false>(const FwdParams, int);  \
   template __global__ void mfma_fwd_kernel<T, 256, 1, true, false, true>(const FwdParams, int);
@@ -697,11 +437,10 @@ DK_INSTANTIATE_FWD(f16_t, 64, true)
 // the look-up-table row.
 static int fwd_group(const FwdParams &p) {
   const int ratio = p.Hq / p.Hkv;
-  static const int max_group = getenv("DKERNEL_FWD_GROUP") ? atoi(getenv("DKERNEL_FWD_GROUP")) : 4;
   // a table with one row per q head may differ inside a kv group
   const int same_lut = (p.csr.num_heads == p.Hq && p.Hq != p.Hkv) ? p.csr.group : ratio;
   for (int g = 4; g > 1; g >>= 1)
-    if (g <= max_group && ratio % g == 0 && same_lut % g == 0) return g;
+    if (ratio % g == 0 && same_lut % g == 0) return g;
   return 1;
 }
 
@@ -738,31 +477,20 @@ bool mfma_fwd_supported(const FwdParams &p, int dtype) {
          p.scale_log2 > 0.f;  // the row maximum is taken before scaling (a scale <= 0 runs on the generic kernels)
 }
 
+// Several q heads per workgroup (G = 2 or 4 heads that share a kv head and a table row).
 template <typename T, int D, int G, bool PAD>
 static int launch_tdg(const FwdParams &p, dim3 grid, int tiles_y, hipStream_t stream) {
   constexpr int smem = 2 * FwdSmem<D>::kStage;
   DK_ALLOW_DYNAMIC_LDS((mfma_fwd_kernel<T, D, G, PAD, false>), smem);
   grid.x = p.Hq / G;
   if (int rc = launch_item_offsets(p, false, stream)) return rc;
-  // One head per workgroup and one q tile (row pairs switched off): one wave per SIMD, where
-  // the software-pipelined kernel is the faster one.  With two waves per SIMD it is not: it
-  // needs more registers than the 256 a wave gets, and spilled loader state is reloaded
-  // between tile requests.  DKERNEL_FWD_PIPE=0 switches it off (A/B measurements).
-  static const bool pipe = !(getenv("DKERNEL_FWD_PIPE") && atoi(getenv("DKERNEL_FWD_PIPE")) == 0);
-  if constexpr (G == 1) if (pipe) {
-    DK_ALLOW_DYNAMIC_LDS((mfma_fwd_pipe_kernel<T, D, G, PAD>), smem);
-    hipLaunchKernelGGL((mfma_fwd_pipe_kernel<T, D, G, PAD>), grid, dim3(128 * G), smem, stream, p, tiles_y);
-    DK_HIP_CHECK(hipGetLastError());
-    return DK_OK;
-  }
   hipLaunchKernelGGL((mfma_fwd_kernel<T, D, G, PAD, false>), grid, dim3(128 * G), smem, stream, p, tiles_y);
   DK_HIP_CHECK(hipGetLastError());
   return DK_OK;
 }
 
-// One head per workgroup: two adjacent q tiles of
-// a head share a workgroup (and the K/V tiles their rows have in common), which gives the two
-// waves per SIMD that a single 64-row tile cannot.  DKERNEL_FWD_ROWPAIR=0 switches it off.
+// One head per workgroup: two adjacent q tiles of a head share a workgroup (and the K/V tiles
+// their rows have in common), which gives the two waves per SIMD that a single 64-row tile cannot.
 template <typename T, int D, bool PAD>
 static int launch_row_pairs(const FwdParams &p, hipStream_t stream) {
   const SeqView &s = p.seqs;
@@ -789,15 +517,10 @@ static int launch_row_pairs(const FwdParams &p, hipStream_t stream) {
 
 template <typename T, int D, bool PAD>
 static int launch_tdp(const FwdParams &p, dim3 grid, int tiles_y, hipStream_t stream) {
-  static const bool row_pairs = !(getenv("DKERNEL_FWD_ROWPAIR") && atoi(getenv("DKERNEL_FWD_ROWPAIR")) == 0);
-  if (row_pairs && fwd_group(p) == 1) return launch_row_pairs<T, D, PAD>(p, stream);
+  if (fwd_group(p) == 1) return launch_row_pairs<T, D, PAD>(p, stream);
   // 64-wide tiles: workgroups of 2 heads (4 waves), three of them per CU, beat one of 4 heads
   const int group = D == 64 && fwd_group(p) == 4 ? 2 : fwd_group(p);
-  switch (group) {
-    case 4: return launch_tdg<T, D, 4, PAD>(p, grid, tiles_y, stream);
-    case 2: return launch_tdg<T, D, 2, PAD>(p, grid, tiles_y, stream);
-    default: return launch_tdg<T, D, 1, PAD>(p, grid, tiles_y, stream);
-  }
+  return group == 4 ? launch_tdg<T, D, 4, PAD>(p, grid, tiles_y, stream) : launch_tdg<T, D, 2, PAD>(p, grid, tiles_y, stream);
 }
 
 // Tables whose entries carry a bit mask over the pattern's 16- or 32-token blocks inside each
@@ -838,13 +561,11 @@ static int launch_256_g(const FwdParams &p, dim3 grid, int tiles_y, hipStream_t 
 
 template <typename T>
 static int launch_256(const FwdParams &p, dim3 grid, int tiles_y, hipStream_t stream) {
-  const bool two = fwd_group(p) >= 2;
   if (p.csr.sub_block)  // (with the mask registers two heads per workgroup would spill)
     return launch_256_g<T, 1, true>(p, grid, tiles_y, stream);
   // one head per workgroup: two adjacent q tiles share the workgroup and their K/V tiles
-  static const bool row_pairs = !(getenv("DKERNEL_FWD_ROWPAIR") && atoi(getenv("DKERNEL_FWD_ROWPAIR")) == 0);
-  if (!two && row_pairs) return launch_row_pairs<T, 256, true>(p, stream);
-  return two ? launch_256_g<T, 2, false>(p, grid, tiles_y, stream) : launch_256_g<T, 1, false>(p, grid, tiles_y, stream);
+  if (fwd_group(p) < 2) return launch_row_pairs<T, 256, true>(p, stream);
+  return launch_256_g<T, 2, false>(p, grid, tiles_y, stream);
 }
 
 // head dims below the tile width (64 or 128) run the zero-padded instantiation

@@ -27,14 +27,11 @@ sys.path.insert(0, ROOT)
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16, vendor figure
 HBM_PEAK_GBS = 8000.0            # MI355X HBM3E, vendor figure
-# HBM bytes per launch, from rocprofv3 --pmc runs of this file (FETCH_SIZE scaled by the copy
-# calibration + WRITE_SIZE; profiles/fwd_bwd_decode_counters.md).  Counters cannot be read from
-# inside this process, so these are quoted, not measured live.
-TRAFFIC_BYTES = {
-    "fwd": 220.9e6 + 136.3e6,
-    "bwd": (611.9e6 + 68.2e6) + (570.1e6 + 134.2e6),   # dQ pass + dK/dV pass
-    "decode": 180.5e6 + 0.3e6,
-}
+# HBM bytes per launch come from rocprofv3 --pmc runs of this file (FETCH_SIZE scaled by the copy
+# calibration + WRITE_SIZE), kept in profiles/hbm_traffic.json together with the library version
+# and the kernels that were profiled.  Counters cannot be read from inside this process, so the
+# figure is quoted, and only while the library still launches those kernels for the workload.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
 BS, LOCAL, VERT, D = 64, 16, 8, 128
 WARM_GPU_SECONDS = 0.3           # untimed calls beyond --warmup until the clocks have settled
 
@@ -95,6 +92,25 @@ def time_steps(fn, steps, warmup):
     return wall, median, marks[0].elapsed_time(marks[steps]) / steps
 
 
+def quoted_traffic(leg, kernels, version):
+    """(bytes per launch or None, note) for `leg` ("fwd", "bwd", "decode"): the profiled figure if it
+    was taken from the kernels that just ran (names and library version agree), else None."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            rec = json.load(f)
+    except (OSError, ValueError) as e:
+        return None, f"no traffic record ({e.__class__.__name__})"
+    kernels = kernels.decode() if isinstance(kernels, bytes) else kernels
+    ent = rec.get(leg)
+    if ent is None:
+        return None, f"no traffic record for {leg}"
+    if rec.get("dk_version") != version:
+        return None, f"traffic record is of library version {rec.get('dk_version')}, this is {version}: re-profile"
+    if ent.get("kernels", "").strip() != kernels.strip():
+        return None, f"traffic record is of kernels '{ent.get('kernels')}', this run launched '{kernels}': re-profile"
+    return float(ent["fetch_bytes"]) + float(ent["write_bytes"]), rec.get("source", TRAFFIC_FILE)
+
+
 def roofline(bound, work, ms, traffic, algorithmic_bytes):
     """work: FLOP (bound "mfma") or bytes (bound "hbm") per launch; ms: median launch duration."""
     if bound == "mfma":
@@ -102,9 +118,9 @@ def roofline(bound, work, ms, traffic, algorithmic_bytes):
     else:
         achieved, peak, unit = work / (ms * 1e-3) / 1e9, HBM_PEAK_GBS, "GB/s"
     return {"bound": bound, "achieved": round(achieved, 2), "peak": peak, "unit": unit,
-            "frac": round(achieved / peak, 4), "traffic": traffic,
-            "traffic_unit": "bytes per launch (rocprofv3 FETCH_SIZE / WRITE_SIZE, separate runs: "
-                            "profiles/fwd_bwd_decode_counters.md)",
+            "frac": round(achieved / peak, 4), "traffic": traffic[0],
+            "traffic_unit": "bytes per launch (rocprofv3 FETCH_SIZE / WRITE_SIZE, separate runs)",
+            "traffic_source": traffic[1],
             "algorithmic_bytes": algorithmic_bytes, "kernel_ms": round(ms, 5)}
 
 
@@ -171,8 +187,10 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"copy_bytes_read": 1 << 30, "copy_bytes_written": 1 << 30, "copies": 3}))
         return
-    from dkernel_amd import LocalStrideSparseAttention, ops
+    from dkernel_amd import LocalStrideSparseAttention, _lib, ops
     ops.set_impl(args.impl)
+    lib = _lib.lib()
+    version = lib.dk_version()
     dev = "cuda:0"
     torch.cuda.set_device(0)
     g = torch.Generator().manual_seed(20)
@@ -187,9 +205,9 @@ def main():
     v = gen((B, L, Hkv, D), g, torch.bfloat16).to(dev)
     with torch.no_grad():
         wall_ms, ev_ms, ev_mean = time_steps(lambda: mod(q, k, v, sm, return_lse=True), args.steps, args.warmup)
+    fwd_kernels = lib.dk_last_kernels().decode()
     flops = block_flops(nnz) * B
     value = flops / (wall_ms * 1e-3) / 1e12
-    auto = args.impl == "auto"
     # q + k + v read once, o + lse written once
     fwd_bytes = (2 * B * L * Hq * D + 2 * B * L * Hkv * D) * 2 + B * L * Hq * 4
 
@@ -202,8 +220,9 @@ def main():
         "config": {"workload": "prefill fwd + LSE: B=2 L=8192 Hq=32 Hkv=8 d=128 bf16, block 64, "
                                "local 16, vert 8, heterogeneous heads, causal",
                    "active_blocks_per_batch": nnz, "flop_per_step": flops, "impl": args.impl},
-        "roofline": roofline("mfma", flops, ev_ms, TRAFFIC_BYTES["fwd"] if auto else None, fwd_bytes),
+        "roofline": roofline("mfma", flops, ev_ms, quoted_traffic("fwd", fwd_kernels, version), fwd_bytes),
     }
+    out["roofline"]["kernels"] = fwd_kernels
     out["roofline"]["kernel_ms_mean"] = round(ev_mean, 5)
     del q, k, v
 
@@ -230,7 +249,9 @@ def main():
                         "tflops": round(bwd_flops / (e2 * 1e-3) / 1e12, 2),
                         "ms": round(e2, 4), "frac_of_mfma_peak":
                         round(bwd_flops / (e2 * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
-                        "roofline": roofline("mfma", bwd_flops, e2, TRAFFIC_BYTES["bwd"] if auto else None, bwd_bytes),
+                        "kernels": ops.last_bwd_kernels.decode(),
+                        "roofline": roofline("mfma", bwd_flops, e2,
+                                             quoted_traffic("bwd", ops.last_bwd_kernels, version), bwd_bytes),
                         "fwd_mha_tflops": round(block_flops(nnz2) / (ef * 1e-3) / 1e12, 2)}
         del q2, k2, v2, do2, o2
         # ---- C3: batched decode over left-padded KV --------------------------
@@ -263,6 +284,7 @@ def main():
                 step[0] += 1
                 return mod(qd, kd, vd, sm, left_paddings=left)
             _, ed_eager, _ = time_steps(decode_step, args.steps, args.warmup)
+            dec_kernels = lib.dk_last_kernels().decode()
             wd = time_loop(decode_step, args.steps, 2)
             # An eager step is bounded by the Python launcher (the GPU idles between steps), so the
             # kernel's own duration is measured on a HIP graph of 8 steps (both K/V sets in turn,
@@ -281,17 +303,22 @@ def main():
                     decode_step()
             _, eg, _ = time_steps(graph.replay, max(10, args.steps), 3)
             ed = eg / 8
+        dec_traffic = quoted_traffic("decode", dec_kernels, version)
         extra["decode"] = {"workload": "32 seqs x 1 token, Hq=32 Hkv=8 d=128 bf16, KV len U[1024,8192] left-padded, "
                                        "2 K/V sets alternated (working set > Infinity Cache)",
-                           "us_per_step": round(wd * 1e3, 2), "kernel_us": round(ed * 1e3, 2),
+                           "us_per_step": round(wd * 1e3, 2), "graph_step_us": round(ed * 1e3, 2),
                            "eager_event_us": round(ed_eager * 1e3, 2),
                            "timing": "us_per_step: eager module calls back to back, wall clock; eager_event_us: the same "
-                                     "with a HIP event between the steps (median); kernel_us: HIP graph of 8 steps, "
-                                     "median replay / 8",
+                                     "with a HIP event between the steps (median); graph_step_us: HIP graph of 8 steps, "
+                                     "median replay / 8 (every kernel of a step, no launch gaps: what rocprofv3 reports as "
+                                     "the kernels' duration)",
+                           "kernels": dec_kernels,
                            "algorithmic_MB": round(byts / 1e6, 2),
                            "achieved_GBs": round(byts / (ed * 1e-3) / 1e9, 1),
                            "frac_of_hbm_peak": round(byts / (ed * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                           "roofline": roofline("hbm", byts, ed, TRAFFIC_BYTES["decode"] if auto else None, byts)}
+                           "roofline": roofline("hbm", byts, ed, dec_traffic, byts),
+                           "roofline_eager_events": roofline("hbm", byts, ed_eager, dec_traffic, byts)}
+        extra["decode"]["kernel_us"] = extra["decode"]["graph_step_us"]   # former name of the same figure
         out["extra"] = extra
 
     if not args.no_cpu:

@@ -67,6 +67,7 @@ class PagedKV(C.Structure):
 SYMBOLS = {
     "dk_version": (C.c_int, []),
     "dk_last_error": (C.c_char_p, []),
+    "dk_last_kernels": (C.c_char_p, []),
     "dk_local_stride_mask": (C.c_int, [i32] * 14 + [vp]),
     "dk_csr_count": (C.c_int, [vp, i32, i32, i32, i64, i64, i64, vp, C.POINTER(i32)]),
     "dk_csr_fill": (C.c_int, [vp, i32, i32, i32, i64, i64, i64, i32, vp, vp]),

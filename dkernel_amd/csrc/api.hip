@@ -158,12 +158,17 @@ static int make_bwd_params(const dk_bwd_args *a, BwdParams &p, bool &empty) {
 // ---------------------------------------------------------------------------
 static __device__ __align__(256) unsigned char scratch[DK_NOALLOC_SCRATCH_BYTES];
 
-static int static_scratch(void **out) {
+static int static_scratch(hipStream_t stream, void **out) {
   constexpr int kMaxDevices = 64;
   static std::atomic<void *> per_device[kMaxDevices];  // zero-initialised
   int dev = 0;
   DK_HIP_CHECK(hipGetDevice(&dev));
   DK_REQUIRE(dev >= 0 && dev < kMaxDevices, "device ordinal %d beyond %d", dev, kMaxDevices);
+  if (stream) {  // the array of the current device is the one the kernels of this stream can reach
+    hipDevice_t sdev = 0;
+    DK_HIP_CHECK(hipStreamGetDevice(stream, &sdev));
+    DK_REQUIRE((int)sdev == dev, "the stream belongs to device %d but device %d is current", (int)sdev, dev);
+  }
   void *ptr = per_device[dev].load(std::memory_order_acquire);
   if (!ptr) {  // first call on this device (a race between threads only repeats the lookup)
     DK_HIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
@@ -193,7 +198,7 @@ int dk_fwd_noalloc(const dk_fwd_args *a) {
              (size_t)DK_NOALLOC_SCRATCH_BYTES);
   if (need > 0) {
     void *ptr = nullptr;
-    if (int rc = static_scratch(&ptr)) return rc;
+    if (int rc = static_scratch((hipStream_t)a->stream, &ptr)) return rc;
     b.workspace = ptr;
     b.workspace_bytes = (size_t)DK_NOALLOC_SCRATCH_BYTES;
   }
@@ -210,6 +215,7 @@ size_t dk_fwd_workspace_bytes(const dk_fwd_args *a) {
 
 int dk_fwd(const dk_fwd_args *a) {
   clear_error();
+  clear_kernels();
   FwdParams p;
   int rc = make_fwd_params(a, p);
   if (rc) return rc;
@@ -241,6 +247,7 @@ size_t dk_bwd_workspace_bytes(const dk_bwd_args *a) {
 
 int dk_fwd_paged(const dk_fwd_args *a, const dk_paged_kv *pg) {
   clear_error();
+  clear_kernels();
   DK_REQUIRE(pg != nullptr && pg->block_table != nullptr, "page table is NULL");
   DK_REQUIRE(pg->page_size >= 16 && is_pow2(pg->page_size), "page_size must be a power of two >= 16, got %d",
              pg->page_size);
@@ -275,6 +282,7 @@ int dk_fwd_paged(const dk_fwd_args *a, const dk_paged_kv *pg) {
 
 int dk_bwd(const dk_bwd_args *a) {
   clear_error();
+  clear_kernels();
   BwdParams p;
   bool empty;
   const int rc = make_bwd_params(a, p, empty);

@@ -16,6 +16,13 @@ namespace dk {
 int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 void clear_error();
 
+// Names of the kernels that the current forward / backward call has launched on this thread
+// (dk_last_kernels()): `kernel` plus the template arguments of the launcher that chose it, taken
+// from its __PRETTY_FUNCTION__.  Tests and the benchmark use it to tell which path ran.
+void note_kernel(const char *kernel, const char *launcher_signature);
+void clear_kernels();
+#define DK_NOTE_KERNEL(kernel) ::dk::note_kernel(kernel, __PRETTY_FUNCTION__)
+
 #define DK_REQUIRE(cond, ...)                                   \
   do {                                                          \
     if (!(cond)) return ::dk::fail(DK_ERR_INVALID, __VA_ARGS__); \

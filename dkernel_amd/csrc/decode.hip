@@ -525,10 +525,12 @@ static int launch_decode_td(const FwdParams &p, float *ws, hipStream_t stream) {
   DK_REQUIRE(groups <= 65535, "too many decode units");
   DK_REQUIRE(smem <= 160 * 1024, "decode workgroup needs %d bytes of LDS", smem);
   DK_ALLOW_DYNAMIC_LDS((decode_partial_kernel<T, D, PAD, SUB, PAGED, KV8, W>), smem);
+  DK_NOTE_KERNEL("decode_partial_kernel");
   hipLaunchKernelGGL((decode_partial_kernel<T, D, PAD, SUB, PAGED, KV8, W>), dim3(groups, p.Hkv, p.seqs.batch),
                      dim3(64 * W), smem, stream, p, ws, unit_blocks, max_units);
   DK_HIP_CHECK(hipGetLastError());
   if (groups == 1) return DK_OK;  // every row was finished inside its workgroup
+  DK_NOTE_KERNEL("decode_combine_kernel");
   hipLaunchKernelGGL((decode_combine_kernel<T, D, PAD>), dim3(p.Hq, p.seqs.batch), dim3(64), 0, stream, p, ws,
                      unit_blocks, max_units, W);
   DK_HIP_CHECK(hipGetLastError());

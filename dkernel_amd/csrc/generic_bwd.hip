@@ -312,6 +312,7 @@ template <typename T, int DPAD>
 static int launch_bwd_td(const BwdParams &p, hipStream_t stream) {
   constexpr int R = 256 / (DPAD / 32);
   const SeqView &s = p.seqs;
+  DK_NOTE_KERNEL("generic_delta_kernel");
   hipLaunchKernelGGL((generic_delta_kernel<T, DPAD>), dim3(cdiv(s.max_q_len, R), p.Hq, s.batch), dim3(256), 0,
                      stream, p);
   DK_HIP_CHECK(hipGetLastError());
@@ -320,6 +321,7 @@ static int launch_bwd_td(const BwdParams &p, hipStream_t stream) {
     const int rows_wg = BM < R ? BM : R;
     const int past = p.causal ? s.max_k_len - s.max_q_len : 0;
     const int blocks = (past + s.max_q_len - 1) / BM - past / BM + 1;
+    DK_NOTE_KERNEL("generic_dq_kernel");
     hipLaunchKernelGGL((generic_dq_kernel<T, DPAD>), dim3(blocks * (BM / rows_wg), p.Hq, s.batch), dim3(256), 0,
                        stream, p);
     DK_HIP_CHECK(hipGetLastError());
@@ -327,6 +329,7 @@ static int launch_bwd_td(const BwdParams &p, hipStream_t stream) {
   {
     const int BN = p.csc.block_rows;
     const int keys_wg = BN < R ? BN : R;
+    DK_NOTE_KERNEL("generic_dkdv_kernel");
     hipLaunchKernelGGL((generic_dkdv_kernel<T, DPAD>),
                        dim3(cdiv(s.max_k_len, BN) * (BN / keys_wg), p.Hkv, s.batch), dim3(256), 0, stream, p);
     DK_HIP_CHECK(hipGetLastError());

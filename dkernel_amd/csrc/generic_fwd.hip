@@ -154,6 +154,7 @@ __global__ __launch_bounds__(256) void generic_fwd_kernel(const FwdParams p) {
 template <typename T>
 static int launch_generic_fwd_t(const FwdParams &p, dim3 grid_for[3], hipStream_t stream) {
   const int dpad = p.D <= 64 ? 64 : (p.D <= 128 ? 128 : 256);
+  DK_NOTE_KERNEL(dpad == 64 ? "generic_fwd_kernel<64>" : dpad == 128 ? "generic_fwd_kernel<128>" : "generic_fwd_kernel<256>");
   if (dpad == 64)
     hipLaunchKernelGGL((generic_fwd_kernel<T, 64>), grid_for[0], dim3(256), 0, stream, p);
   else if (dpad == 128)

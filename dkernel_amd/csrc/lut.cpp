@@ -20,6 +20,16 @@ int fail(int code, const char *fmt, ...) {
 }
 void clear_error() { g_err[0] = 0; }
 
+static thread_local char g_kernels[1024] = "";
+
+void clear_kernels() { g_kernels[0] = 0; }
+void note_kernel(const char *kernel, const char *launcher_signature) {
+  // "... launcher(args) [T = dk::bf16_t, D = 128, ...]" -> "kernel [T = dk::bf16_t, D = 128, ...]; "
+  const char *args = launcher_signature ? strrchr(launcher_signature, '[') : nullptr;
+  const size_t used = strlen(g_kernels);
+  snprintf(g_kernels + used, sizeof(g_kernels) - used, "%s%s%s; ", kernel, args ? " " : "", args ? args : "");
+}
+
 }  // namespace dk
 
 using dk::fail;
@@ -28,6 +38,7 @@ extern "C" {
 
 int dk_version(void) { return 300; /* 0.3.0 */ }
 const char *dk_last_error(void) { return dk::g_err; }
+const char *dk_last_kernels(void) { return dk::g_kernels; }
 
 // dkernel/utils.py:157-215.  Head h of the pattern belongs to kv head
 // h / (num_heads / num_kv_heads); kv heads >= num_kv_heads - num_dense_heads

@@ -858,6 +858,7 @@ static int launch_bwd_td(const BwdParams &p, void *workspace, size_t workspace_b
   const int cblocks = cdiv(s.max_k_len, 64);
   DK_REQUIRE(tiles <= 65535 && cblocks <= 65535, "sequence too long for one launch");
   // dQ first: it also writes delta, which the dK/dV pass reads
+  DK_NOTE_KERNEL("mfma_dq_kernel");
   hipLaunchKernelGGL((mfma_dq_kernel<T, D, PAD, SUB>), dim3(p.Hq, tiles, s.batch), dim3(256), smem_dq, stream, p, tiles);
   DK_HIP_CHECK(hipGetLastError());
   // With several q heads per kv head a workgroup per kv head walks all of them, and the longest
@@ -871,14 +872,17 @@ static int launch_bwd_td(const BwdParams &p, void *workspace, size_t workspace_b
     float *part_k = (float *)workspace, *part_v = part_k + (int64_t)s.batch * p.Hq * keys * p.D;
     pp.dk = TensorView{part_k, p.Hq * keys * p.D, keys * p.D, p.D};
     pp.dv = TensorView{part_v, p.Hq * keys * p.D, keys * p.D, p.D};
+    DK_NOTE_KERNEL("mfma_dkdv_kernel (one workgroup per q head)");
     hipLaunchKernelGGL((mfma_dkdv_kernel<T, D, PAD, SUB>), dim3(p.Hq, cblocks, s.batch), dim3(256), smem_dkdv, stream, pp, 1);
     DK_HIP_CHECK(hipGetLastError());
     const int64_t total = (int64_t)s.batch * p.Hkv * keys * (p.D / 8);
+    DK_NOTE_KERNEL("dkdv_group_sum_kernel");
     hipLaunchKernelGGL((dkdv_group_sum_kernel<T>), dim3((unsigned)cdiv64(total, 256), 2), dim3(256), 0, stream, part_k,
                        part_v, p.dk, p.dv, s.batch, p.Hq, p.Hkv, (int)keys, p.D);
     DK_HIP_CHECK(hipGetLastError());
     return DK_OK;
   }
+  DK_NOTE_KERNEL("mfma_dkdv_kernel");
   hipLaunchKernelGGL((mfma_dkdv_kernel<T, D, PAD, SUB>), dim3(p.Hkv, cblocks, s.batch), dim3(256), smem_dkdv, stream, p, 0);
   DK_HIP_CHECK(hipGetLastError());
   return DK_OK;

@@ -408,6 +408,10 @@ __device__ __forceinline__ void store_tile_rows(char *stage, const floatx16 (&ac
           pack4<T>(acc[dt][r4 * 4] * row_scale, acc[dt][r4 * 4 + 1] * row_scale, acc[dt][r4 * 4 + 2] * row_scale,
                    acc[dt][r4 * 4 + 3] * row_scale);
     }
+  // The rows read back below were written by other lanes of this wave: LDS operations of a wave
+  // execute in order, so no hardware wait is needed, but the compiler must not move the reads
+  // above the writes (it cannot prove the swizzled addresses disjoint today; this says so).
+  asm volatile("" ::: "memory");
   store_staged_rows<T, D, PAD, 32>(stage, g_row0, row_stride, lane, row_lo, row_hi, real_d);
 }
 

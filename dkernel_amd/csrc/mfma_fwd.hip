@@ -459,6 +459,7 @@ static int launch_item_offsets(const FwdParams &p, bool pairs, hipStream_t strea
   if (!p.seqs.packed || !p.seqs.item_offsets) return DK_OK;
   SeqView s = p.seqs;
   s.item_offsets = nullptr;
+  DK_NOTE_KERNEL("packed_item_offsets_kernel");
   hipLaunchKernelGGL(packed_item_offsets_kernel, dim3(1), dim3(1024), 0, stream, s, p.causal, pairs ? 1 : 0,
                      p.seqs.item_offsets);
   DK_HIP_CHECK(hipGetLastError());
@@ -484,6 +485,7 @@ static int launch_tdg(const FwdParams &p, dim3 grid, int tiles_y, hipStream_t st
   DK_ALLOW_DYNAMIC_LDS((mfma_fwd_kernel<T, D, G, PAD, false>), smem);
   grid.x = p.Hq / G;
   if (int rc = launch_item_offsets(p, false, stream)) return rc;
+  DK_NOTE_KERNEL("mfma_fwd_kernel");
   hipLaunchKernelGGL((mfma_fwd_kernel<T, D, G, PAD, false>), grid, dim3(128 * G), smem, stream, p, tiles_y);
   DK_HIP_CHECK(hipGetLastError());
   return DK_OK;
@@ -509,6 +511,7 @@ static int launch_row_pairs(const FwdParams &p, hipStream_t stream) {
   }
   DK_REQUIRE(pairs <= 65535, "too many q tiles for one launch (%d)", pairs);
   if (int rc = launch_item_offsets(p, true, stream)) return rc;
+  DK_NOTE_KERNEL("mfma_fwd_kernel");
   hipLaunchKernelGGL((mfma_fwd_kernel<T, D, 2, PAD, true>), dim3(p.Hq, pairs, s.packed ? 1 : s.batch), dim3(256), smem,
                      stream, p, pairs);
   DK_HIP_CHECK(hipGetLastError());
@@ -531,6 +534,7 @@ static int launch_sub_g(const FwdParams &p, dim3 grid, int tiles_y, hipStream_t 
   DK_ALLOW_DYNAMIC_LDS((mfma_fwd_kernel<T, D, G, PAD, false, true>), smem);
   grid.x = p.Hq / G;
   if (int rc = launch_item_offsets(p, false, stream)) return rc;
+  DK_NOTE_KERNEL("mfma_fwd_kernel");
   hipLaunchKernelGGL((mfma_fwd_kernel<T, D, G, PAD, false, true>), grid, dim3(128 * G), smem, stream, p, tiles_y);
   DK_HIP_CHECK(hipGetLastError());
   return DK_OK;
@@ -554,6 +558,7 @@ static int launch_256_g(const FwdParams &p, dim3 grid, int tiles_y, hipStream_t 
   DK_ALLOW_DYNAMIC_LDS((mfma_fwd_kernel<T, 256, G, true, false, SUB>), smem);
   grid.x = p.Hq / G;
   if (int rc = launch_item_offsets(p, false, stream)) return rc;
+  DK_NOTE_KERNEL("mfma_fwd_kernel");
   hipLaunchKernelGGL((mfma_fwd_kernel<T, 256, G, true, false, SUB>), grid, dim3(128 * G), smem, stream, p, tiles_y);
   DK_HIP_CHECK(hipGetLastError());
   return DK_OK;

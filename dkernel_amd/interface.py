@@ -17,7 +17,7 @@ from torch import Tensor
 from .ops import _sparse_attention
 from .utils import (dense_to_ccol_row, dense_to_crow_col, get_sparse_attn_mask, is_kv_cache_efficient,
                     masked_tile_tables, merge_split_fwd_kernel_blocks, multiple_of, split_tile_tables,
-                    tile_sizes_keep_pattern,
+                    merged_rows_pattern, tile_sizes_keep_pattern,
                     verify_sparse_pattern, zero_stride)
 
 _KERNEL_TILE = 64  # q and k tile of the matrix-core kernels
@@ -58,11 +58,12 @@ class SparseAttention(torch.nn.Module):
         block_n = block_size; the attributes and the `layout_*` buffers follow
         these values as in the reference.  The kernels themselves read extra
         tables built for their 64 x 64 tiles (`kernel_*`: larger blocks split;
-        `masked_*`: smaller blocks as tiles with a bit mask; `exact_csr_*`:
-        unmerged tiles), which follow the pattern exactly -- unless block_m is
+        `masked_*`: smaller blocks as tiles with a bit mask; `exact_*`:
+        unmerged tiles), which follow the pattern exactly.  When block_m is
         given and merging q rows widens the pattern (a later pattern row of a
-        merged tile holds a column an earlier one lacks): then the merged table
-        is used as given, on the generic kernels.
+        merged tile holds a column an earlier one lacks, and the reference's
+        merged table lets the earlier rows attend it too), those tables are
+        built from the widened pattern: the result is that of the merged table.
     kwargs: "out" (output tensor), "d_splits" (accepted, unused), "inference"
         (skip saving the log-sum-exp for backward; default: no input needs grad).
 
@@ -125,11 +126,18 @@ class SparseAttention(torch.nn.Module):
             assert self.block_n <= block_size
 
         # Tile sizes given by the caller are honoured in the layout_* buffers.  The kernels run
-        # 64 x 64 tiles of their own (below) whenever that attends the same blocks, i.e. always
-        # except for a merged-row table over a pattern in which a later row of a merged tile
-        # holds a column that an earlier one lacks.
-        own_tiles = not explicit_tiles or tile_sizes_keep_pattern(block_size, sparse_pattern, self.block_m,
-                                                                  self.block_n, causal)
+        # 64 x 64 tiles of their own (below), which attend the same blocks.
+        # (a merged-row table over a pattern that it widens: the kernels' own tiles then follow
+        # the widened pattern, block by block what the merged table attends)
+        kernel_pattern = sparse_pattern
+        if explicit_tiles and not tile_sizes_keep_pattern(block_size, sparse_pattern, self.block_m, self.block_n,
+                                                          causal):
+            kernel_pattern = merged_rows_pattern(block_size, sparse_pattern, self.block_m, self.block_n,
+                                                 causal).to(sparse_pattern.device)
+            if kernel_pattern.size(0) == 1:
+                kernel_pattern = zero_stride(kernel_pattern)
+        widened = kernel_pattern is not sparse_pattern
+        own_tiles = True
         # patterns with blocks larger than the 64 x 64 tile of the matrix-core kernels run on
         # tables split to that tile
         split_for_kernels = own_tiles and block_size > _KERNEL_TILE
@@ -163,7 +171,7 @@ class SparseAttention(torch.nn.Module):
         # The layout_* buffers keep the reference's shapes; the kernels read these when present.
         self.kernel_tile = None
         if split_for_kernels:
-            tile_csr, tile_csc = split_tile_tables(block_size, sparse_pattern, _KERNEL_TILE, causal=causal)
+            tile_csr, tile_csc = split_tile_tables(block_size, kernel_pattern, _KERNEL_TILE, causal=causal)
             tile_csr, tile_csc = list(tile_csr), list(tile_csc)
             if tile_csr[0].size(0) == 1:
                 tile_csr = [zero_stride(x) for x in tile_csr]
@@ -183,8 +191,9 @@ class SparseAttention(torch.nn.Module):
         # layout_csr_* buffers keep that table; the kernels follow the pattern itself: unmerged
         # tiles for the generic kernels, masked 64 x 64 tiles for the matrix-core kernels.
         self.exact_tile = None
+        self.exact_csc = False
         if own_tiles and not split_for_kernels and (self.block_m != block_size or self.block_n != block_size):
-            exact = list(dense_to_crow_col(sparse_pattern))
+            exact = list(dense_to_crow_col(kernel_pattern))
             if exact[0].dim() == 1:
                 exact = [x[None] for x in exact]
             if exact[0].size(0) == 1:
@@ -195,10 +204,19 @@ class SparseAttention(torch.nn.Module):
             self.kwargs['lut_max_row'] = self.lut_max_row
             self.register_buffer("exact_csr_crow", exact[0].to(torch.int32), persistent=False)
             self.register_buffer("exact_csr_col", exact[1].to(torch.int32), persistent=False)
+            if widened:  # the column walk of the backward follows the widened pattern as well
+                exact_c = list(dense_to_ccol_row(kernel_pattern, include_values=False))
+                if exact_c[0].dim() == 1:
+                    exact_c = [x[None] for x in exact_c]
+                if exact_c[0].size(0) == 1:
+                    exact_c = [zero_stride(x) for x in exact_c]
+                self.exact_csc = True
+                self.register_buffer("exact_csc_ccol", exact_c[0].to(torch.int32), persistent=False)
+                self.register_buffer("exact_csc_row", exact_c[1].to(torch.int32), persistent=False)
 
         self.mask_tile = None
         if mask_for_kernels:
-            m_csr, m_csc = masked_tile_tables(block_size, sparse_pattern, _KERNEL_TILE)
+            m_csr, m_csc = masked_tile_tables(block_size, kernel_pattern, _KERNEL_TILE)
             m_csr, m_csc = list(m_csr), list(m_csc)
             if m_csr[0].size(0) == 1:
                 m_csr = [zero_stride(x) for x in m_csr]
@@ -250,6 +268,8 @@ class SparseAttention(torch.nn.Module):
             layout_csc = (self.layout_csc_ccol, self.layout_csc_row, self.block_m2, self.block_n2)
             if self.exact_tile is not None:
                 layout_csr = (self.exact_csr_crow, self.exact_csr_col, self.exact_tile, self.exact_tile)
+                if self.exact_csc:
+                    layout_csc = (self.exact_csc_ccol, self.exact_csc_row, self.exact_tile, self.exact_tile)
         if self.mask_tile is not None:
             # (crow, (col, mask), tile rows, tile cols, pattern block size), longest row
             kwargs["masked_layouts"] = ((self.masked_csr_crow, self.masked_csr_col, self.mask_tile,

@@ -89,15 +89,18 @@ _LUT_CACHE = {}
 
 def _lut(layout: Tuple[Tensor, Tensor, int, int], device, group: int = 1, max_row: int = 0) -> _lib.Lut:
     """dk_lut of a layout tuple.  The descriptor of a module's tables never changes, so it is
-    built once per (tables, hints) and copied from then on (a decode step's host time counts)."""
-    key = (layout[0].data_ptr(), layout[1].data_ptr(), layout[0].shape, layout[1].shape, layout[0].stride(),
-           layout[1].stride(), tuple(int(x) for x in layout[2:]), device, group, max_row)
+    built (and checked) once per (tables, hints) and copied from then on (a decode step's host
+    time counts).  An entry keeps its two tensors alive, so their addresses cannot be handed to
+    other tensors while the entry exists; the caller gets a copy of its own."""
+    key = (layout[0].data_ptr(), layout[1].data_ptr(), layout[0].dtype, layout[1].dtype, layout[0].shape,
+           layout[1].shape, layout[0].stride(), layout[1].stride(), tuple(int(x) for x in layout[2:]), device, group,
+           max_row)
     hit = _LUT_CACHE.get(key)
     if hit is None:
         if len(_LUT_CACHE) > 256:
             _LUT_CACHE.clear()
-        hit = _LUT_CACHE[key] = _make_lut(layout, device, group, max_row)
-    return hit
+        hit = _LUT_CACHE[key] = (_make_lut(layout, device, group, max_row), layout[0], layout[1])
+    return _lib.Lut.from_buffer_copy(hit[0])
 
 
 def _make_lut(layout: Tuple[Tensor, Tensor, int, int], device, group: int = 1, max_row: int = 0) -> _lib.Lut:
@@ -158,6 +161,7 @@ def _as_i32(x: Tensor, device) -> Tensor:
 
 
 last_fwd_workspace_bytes = 0  # scratch the library asked for in the latest forward (non-zero: split-KV decode)
+last_bwd_kernels = b""        # dk_last_kernels() after the latest backward
 
 
 def _run_fwd(args: _lib.FwdArgs, device) -> None:
@@ -274,6 +278,8 @@ def _backward(ctx, do: Tensor, dlse: Optional[Tensor],
         ws = torch.empty(need, dtype=torch.uint8, device=q.device)
         args.workspace, args.workspace_bytes = ws.data_ptr(), need
     _lib.check(lib.dk_bwd(C.byref(args)))
+    global last_bwd_kernels
+    last_bwd_kernels = lib.dk_last_kernels()  # (backward runs on an autograd thread; the list is per thread)
     return dq, dk, dv
 
 
@@ -530,6 +536,10 @@ class _sparse_attention(torch.autograd.Function):
         # Patterns with blocks below the kernel tile run on the masked tile tables whenever the
         # matrix-core kernels take these inputs (the backward decides again for its own tensors).
         masked = kwargs.get("masked_layouts", None)
+        if masked is not None and sm_scale <= 0:
+            # the matrix-core forward takes row maxima before scaling (scale > 0) and only it reads
+            # masked tiles: other scales run forward and backward on the unmasked tables
+            masked = None
         ctx.masked_layouts = masked
         if masked is not None and _matrix_core_applies(q, k, v, kwargs.get("out", None)):
             layout_csr, _, lut_max_row = masked

@@ -274,6 +274,29 @@ def tile_sizes_keep_pattern(block_size: int, sparse_pattern: Tensor, block_m: in
     return bool(((eff == own) | ~visible[None]).all())
 
 
+def merged_rows_pattern(block_size: int, sparse_pattern: Tensor, block_m: int, block_n: int,
+                        causal: bool = True) -> Tensor:
+    """The block pattern that a table of block_m x block_n kernel tiles attends, at the pattern's
+    own granularity: with merged q rows (block_m > block_size) every pattern row of a merged tile
+    up to the last one that holds a column attends that column (rows at or beyond micro_M are
+    excluded, dkernel/utils.py:299-308; dkernel/ops/sparse_attn_fwd.py:113-134), so a column held
+    only by a later row widens the rows before it.  Blocks entirely above the token diagonal stay
+    out when causal.  Without merging this is the pattern itself."""
+    p = (sparse_pattern != 0).to("cpu")
+    out, merged = _tile_pattern(block_size, sparse_pattern, block_m, block_n, causal)
+    if not merged:
+        return p.to(torch.uint8)
+    H, M, N = p.shape
+    mm, split_n = block_m // block_size, block_size // block_n
+    om, on = out.shape[1:]
+    sub = torch.arange(mm)[None, None, :, None] * block_size
+    eff = (out[:, :, None, :] > sub).reshape(H, om * mm, on)[:, :M]   # (H, M, column tiles)
+    wide = eff[:, :, ::split_n][:, :, :N]                              # first column tile of each block
+    if causal:
+        wide = wide & (torch.arange(N)[None, :] <= torch.arange(M)[:, None])[None]
+    return wide.to(torch.uint8)
+
+
 def split_tile_tables(block_size: int, sparse_pattern: Tensor, tile: int,
                       causal: bool = True) -> Tuple[Tuple[Tensor, Tensor], Tuple[Tensor, Tensor]]:
     """CSR and CSC tables of a pattern whose blocks are split into tile x tile

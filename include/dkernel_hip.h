@@ -31,6 +31,10 @@ enum dk_impl { DK_IMPL_AUTO = 0, DK_IMPL_GENERIC = 1, DK_IMPL_MFMA = 2 };
 
 int dk_version(void);              /* 10000*major + 100*minor + patch */
 const char *dk_last_error(void);   /* thread-local, never NULL */
+/* Kernels that the latest dk_fwd / dk_fwd_paged / dk_fwd_noalloc / dk_bwd call on this thread
+ * launched, "name [template arguments]; " each, in launch order (thread-local, never NULL).  No
+ * counterpart in the reference; tests and bench.py use it to tell which path a call took. */
+const char *dk_last_kernels(void);
 
 /* --------------------------------------------------------------------------
  * Host side: layout / look-up-table builder (runs on the CPU, no GPU needed)
@@ -175,7 +179,10 @@ size_t dk_fwd_workspace_bytes(const dk_fwd_args *args);
  * scratch are refused with DK_ERR_INVALID (dk_fwd_workspace_bytes tells how much a call needs).
  * Each GPU holds one such array for the life of the process and every call on that GPU uses it:
  * calls that overlap on one GPU (two streams, two threads) race on it -- serialise them or use
- * dk_fwd with separate workspaces.  No counterpart in the reference, whose launchers allocate
+ * dk_fwd with separate workspaces.  The device that owns args->stream must be the current one.
+ * Before a call is recorded into a HIP graph, make one ordinary call with the same kind of
+ * arguments on that device: the first call looks up the array's address and raises the kernels'
+ * LDS limits, which a capturing stream does not allow.  No counterpart in the reference, whose launchers allocate
  * with torch on every call (dkernel/ops/sparse_attn_inference.py:67,230). */
 #define DK_NOALLOC_SCRATCH_BYTES (8u << 20)
 int dk_fwd_noalloc(const dk_fwd_args *args);

@@ -145,6 +145,28 @@ def test_negative_softmax_scale(D):
     assert_close("LSE", lse, rl, atol=LSE_TOL, rtol=0)
 
 
+@pytest.mark.parametrize("bs", [16, 32])
+def test_negative_softmax_scale_small_blocks(bs):
+    """Pattern blocks below the kernel tile normally run on masked 64 x 64 tiles, which only the
+    matrix-core kernels read; with a scale <= 0 forward and backward take the unmasked tables."""
+    B, H, L, D = 1, 2, 200, 64
+    q, k, v, do = make_qkv(B, L, L, H, H, D, torch.bfloat16, with_do=True)
+    bm = expand_heads(OL.block_mask(H, 256, bs, 3, 4), H)
+    qo, ko, vo = (x.float().requires_grad_() for x in (q, k, v))
+    ro, rl = oracle_fwd(qo, ko, vo, bm, bs, -0.05)
+    ro.backward(do.float())
+    mod = New(H, 256, bs, 3, 4).to(DEV)
+    assert mod.mask_tile == 64
+    qd, kd, vd = (x.to(DEV).requires_grad_() for x in (q, k, v))
+    out, lse = mod(qd, kd, vd, -0.05, return_lse=True)
+    out.backward(do.to(DEV))
+    assert_close("O", out, ro, **TOL)
+    assert_close("LSE", lse, rl, atol=LSE_TOL, rtol=0)
+    assert_close("dQ", qd.grad, qo.grad, **TOL)
+    assert_close("dK", kd.grad, ko.grad, **TOL)
+    assert_close("dV", vd.grad, vo.grad, **TOL)
+
+
 @pytest.mark.parametrize("past", [37, 64, 200])
 @pytest.mark.parametrize("Hq,Hkv,D,dtype", [(4, 4, 128, torch.bfloat16), (4, 2, 64, torch.float16), (2, 2, 96, torch.bfloat16)])
 def test_backward_with_more_keys_than_queries(impl, past, Hq, Hkv, D, dtype):
@@ -202,3 +224,24 @@ def test_head_dims_above_128_on_the_matrix_cores(D, bs, Hq, Hkv, dtype):
     assert_close("dV", vd.grad, vo.grad, **TOL)
     assert_close("dK", kd.grad, ko.grad, **TOL)
     assert_close("dQ", qd.grad, qo.grad, **TOL)
+
+
+def test_last_kernels_names_the_path_taken():
+    """dk_last_kernels(): which kernels the latest call launched (what bench.py's traffic guard and
+    this test read)."""
+    lib = ops._lib.lib()
+    L, D = 256, 128
+    sm = 1 / math.sqrt(D)
+    try:
+        for Hq, Hkv, impl, want in ((8, 2, "auto", "mfma_fwd_kernel [T = dk::bf16_t, D = 128, G = 4, PAD = false]; "),
+                                    (2, 2, "auto", "mfma_fwd_kernel [T = dk::bf16_t, D = 128, PAD = false]; "),
+                                    (2, 2, "generic", "generic_fwd_kernel<128> [T = dk::bf16_t]; ")):
+            ops.set_impl(impl)
+            q, k, v = (x.to(DEV) for x in make_qkv(1, L, L, Hq, Hkv, D, torch.bfloat16))
+            New(Hq, L, 64, 2, 3, num_kv_heads=Hkv).to(DEV)(q, k, v, sm)
+            assert lib.dk_last_kernels().decode() == want
+        q.requires_grad_()
+        New(2, L, 64, 2, 3).to(DEV)(q, k, v, sm).sum().backward()
+        assert ops.last_bwd_kernels.decode().startswith("generic_delta_kernel")
+    finally:
+        ops.set_impl("auto")

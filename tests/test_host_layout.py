@@ -244,7 +244,13 @@ def test_tile_sizes_given_by_the_caller_keep_the_pattern_or_not():
     assert U.tile_sizes_keep_pattern(64, pat, 64, 32, True)                 # splitting alone never changes it
     with pytest.warns(UserWarning, match="not efficient for KV cache"):
         mod = SparseAttention(64, pat, block_m=128)
-    assert mod.exact_tile is None and mod.mask_tile is None and mod.kernel_tile is None
+    # the kernels' own tiles follow the widened pattern (row 2 attends column 1 as well), rows and columns
+    assert mod.exact_tile == 64 and mod.exact_csc and mod.mask_tile is None and mod.kernel_tile is None
+    wide = torch.tensor([[1, 0, 0, 0], [1, 1, 0, 0], [0, 1, 1, 0], [0, 1, 1, 1]])
+    assert (U.merged_rows_pattern(64, pat, 128, 64, True)[0] == wide).all()
+    assert mod.exact_csr_crow.flatten().tolist() == [0, 1, 3, 5, 8]
+    assert mod.exact_csc_ccol.flatten().tolist() == [0, 2, 5, 7, 8]
+    assert mod.layout_csr_crow.flatten().tolist() == [0, 2, 5]          # the merged table itself, as asked
     # brute force on random causal patterns: expand the merged table and compare
     rng = np.random.default_rng(3)
     for _ in range(40):
@@ -262,6 +268,8 @@ def test_tile_sizes_given_by_the_caller_keep_the_pattern_or_not():
                         eff[0, i * mm + s, c] = 1
         same = bool((np.tril(eff) == dense).all())
         assert U.tile_sizes_keep_pattern(16, torch.from_numpy(dense), 16 * mm, 16, True) == same
+        # ... and what the merged table attends, block by block
+        assert (U.merged_rows_pattern(16, torch.from_numpy(dense), 16 * mm, 16, True).numpy() == np.tril(eff)).all()
 
 
 def _fake_fwd_args(B=2, Hq=8, Hkv=2, D=128, Lq=1, Lk=2048, dtype=0, max_row=10):

@@ -145,3 +145,46 @@ def test_too_much_scratch_is_refused_before_any_launch():
     assert lib.dk_fwd_workspace_bytes(C.byref(a)) > _lib.DK_NOALLOC_SCRATCH_BYTES
     assert lib.dk_fwd_noalloc(C.byref(a)) == _lib.DK_ERR_INVALID
     assert "bytes of scratch" in lib.dk_last_error().decode()
+
+
+def test_recorded_into_a_graph_after_a_warm_up_call():
+    """The entry point under stream capture (one of the callers it exists for): after one ordinary
+    call, a decode step is recorded into a graph and every replay, with K/V and q rewritten in
+    place between them, must give dk_fwd's bits."""
+    B, Hq, Hkv, Lmax, D = 3, 8, 2, 4096, 128
+    lens = [4096, 3000, 2049]
+    g = torch.Generator().manual_seed(11)
+    mod = LocalStrideSparseAttention(Hq, Lmax, 64, 4, 4, num_kv_heads=Hkv).to(DEV)
+    q = torch.randn(B, 1, Hq, D, generator=g).to(torch.bfloat16).to(DEV)
+    k = torch.randn(B, Lmax, Hkv, D, generator=g).to(torch.bfloat16).to(DEV)
+    v = torch.randn(B, Lmax, Hkv, D, generator=g).to(torch.bfloat16).to(DEV)
+    lens_t = torch.tensor(lens, dtype=torch.int32, device=DEV)
+    left = Lmax - lens_t
+    o = torch.zeros_like(q)
+    lse = torch.zeros((B, Hq, 1), dtype=torch.float32, device=DEV)
+    lib = _lib.lib()
+    a, keep = _decode_args(mod, q, k, v, o, lse, left, lens_t)
+    a.workspace, a.workspace_bytes = None, 0
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):   # the warm-up call, on the stream that will capture
+        a.stream = ops._stream()
+        _lib.check(lib.dk_fwd_noalloc(C.byref(a)))
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        a.stream = ops._stream()
+        _lib.check(lib.dk_fwd_noalloc(C.byref(a)))
+    for rep in range(3):
+        q.copy_(torch.randn(B, 1, Hq, D, generator=g).to(torch.bfloat16))
+        k.copy_(torch.randn(B, Lmax, Hkv, D, generator=g).to(torch.bfloat16))
+        o.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        o_graph, lse_graph = o.clone(), lse.clone()
+        o2 = torch.full_like(q, float("nan"))
+        lse2 = torch.full_like(lse, float("nan"))
+        b, keep2 = _decode_args(mod, q, k, v, o2, lse2, left, lens_t)
+        assert _run_both(b) > 0
+        assert torch.equal(o_graph, o2) and torch.equal(lse_graph, lse2), f"replay {rep} differs from dk_fwd"

@@ -355,6 +355,313 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 
 }
 
 // ---------------------------------------------------------------------------
+// dQ pass, two q tiles per workgroup (tiles of 64 and 128 head dims)
+// ---------------------------------------------------------------------------
+// One workgroup = table rows 2u and 2u + 1 of one q head (128 q rows), 4 waves: wave = 32 q rows
+// of one of the two rows, against all 64 keys of a block (two 32-key halves one after the other,
+// in the same registers).  The workgroup walks the union of its two table rows, merged on the
+// fly from the two sorted rows, and copies every K / V tile once for both: neighbouring rows of
+// the local window share 15 of 16 columns and every vertical column, so the tile traffic from
+// the L2 into LDS (what the one-tile kernel spent a quarter of its time on) is halved; a wave
+// skips the blocks its own row does not hold.  Every wave owns the finished dQ of its rows:
+// nothing is summed across waves at the end.
+template <typename T, int D, bool PAD, bool SUB>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, D == 64 ? 3 : 2))) void mfma_dq_pair_kernel(const BwdParams p,
+                                                                                                      int pairs_y) {
+  using M = Mma<T>;
+  using vec8 = typename M::vec8;
+  using TL = Tile<D>;
+  constexpr int NT = 256;
+  constexpr int KS = D / 16, DT = D / 32;
+  constexpr int STAGE = 2 * TL::kBytes;
+  constexpr int EW = SUB ? 2 : 1;  // ints per table entry
+  extern __shared__ __align__(16) char smem[];
+
+  const SeqInfo sq = load_seq(p.seqs, blockIdx.z, p.causal);
+  if (sq.q_len <= 0) return;
+  const int first_rb = sq.past / 64, last_rb = (sq.past + sq.q_len - 1) / 64;
+  const int u = (first_rb >> 1) + pairs_y - 1 - (int)blockIdx.y;  // longest rows first
+  if (u > (last_rb >> 1)) return;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int ts = wave >> 1, rh = wave & 1;  // which of the two table rows, which half of its 64 q rows
+  const int ra = 2 * u, rb = ra + ts;
+  const int h = blockIdx.x;
+  const int kvh = __builtin_amdgcn_readfirstlane(h / (p.Hq / p.Hkv));  // integer division runs on the VALU
+  const int m = lane & 31, g = lane >> 5;
+  const int row0 = rb * 64 + rh * 32;
+  const int pos = row0 + m;
+  const int qi = pos - sq.past;
+  const bool row_ok = qi >= 0 && qi < sq.q_len;  // (a table row without queries of this sequence: false everywhere)
+  if constexpr (PAD) {  // the slots of the head dims beyond p.D stay zero for the whole kernel
+    zero_tiles<NT>(smem, 2 * STAGE, tid);
+    __syncthreads();
+  }
+
+  // Row data: Q and dO of the 128 rows come in as four tiles by LDS DMA (stage 0: first table
+  // row, stage 1: second), O as 16-byte chunks along the rows, multiplied with the dO chunks in
+  // LDS for delta = rowsum(O * dO) - dLSE.  The first K / V request has to wait until every wave
+  // has taken its fragments out of the stages.
+  constexpr int CPR = D / 8;  // 16-byte chunks per row
+  constexpr int OCH = 128 * CPR / NT;
+  __shared__ float delta_rows[128];
+  float lse_raw = -INFINITY, dlse_raw = 0.f;
+  uint4 oreg[OCH];
+  {
+    TileLoader<D, NT, PAD> qload, doload;
+    qload.init(tid, p.q.st, p.D);
+    doload.init(tid, p.dout.st, p.D);
+    const int qi0 = ra * 64 - sq.past;  // query index of the first of the 128 rows (may be negative)
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2) {
+      const int q0 = qi0 + t2 * 64;
+      const T *qb = (const T *)p.q.ptr + sq.b * p.q.sb + h * p.q.sh + (int64_t)q0 * p.q.st;
+      const T *dob = (const T *)p.dout.ptr + sq.b * p.dout.sb + h * p.dout.sh + (int64_t)q0 * p.dout.st;
+      qload.issue(reinterpret_cast<const char *>(qb), -q0, sq.q_len - q0, smem + t2 * STAGE);
+      doload.issue(reinterpret_cast<const char *>(dob), -q0, sq.q_len - q0, smem + t2 * STAGE + TL::kBytes);
+    }
+    const T *ob = (const T *)p.o.ptr + sq.b * p.o.sb + h * p.o.sh + (int64_t)qi0 * p.o.st;
+#pragma unroll
+    for (int j = 0; j < OCH; ++j) {
+      const int r = tid / CPR + j * (NT / CPR), ch = tid % CPR;
+      oreg[j] = make_uint4(0, 0, 0, 0);
+      if (qi0 + r >= 0 && qi0 + r < sq.q_len && (!PAD || ch * 8 < p.D))
+        oreg[j] = *reinterpret_cast<const uint4 *>(ob + (int64_t)r * p.o.st + ch * 8);
+    }
+    if (row_ok) {
+      lse_raw = p.lse.ptr[sq.b * p.lse.sb + h * p.lse.sh + (int64_t)qi * p.lse.st];
+      if (p.dlse.ptr) dlse_raw = p.dlse.ptr[sq.b * p.dlse.sb + h * p.dlse.sh + (int64_t)qi * p.dlse.st];
+    }
+  }
+
+  // the two table rows: entries [e0, emid) are row 2u, [emid, e1) row 2u + 1 (consecutive rows
+  // follow each other in the table); a row without queries of this sequence contributes nothing
+  const int lh = lut_head(p.csr, h, p.Hq, p.Hkv);
+  int e0 = 0, emid = 0, e1 = 0;
+  {
+    const int32_t *rp = p.csr.ptr + lh * p.csr.ptr_sh;
+    if (ra < p.csr.num_rows) scalar_load2(rp + ra, rp + ra + 1, e0, emid);
+    e1 = emid;
+    if (ra + 1 < p.csr.num_rows) e1 = scalar_load(rp + ra + 2);
+    if (ra < first_rb) e0 = emid;
+    if (ra + 1 > last_rb) e1 = emid;
+  }
+  const int32_t *cols = p.csr.idx + lh * p.csr.idx_sh;
+  const T *kbase = (const T *)p.k.ptr + sq.b * p.k.sb + kvh * p.k.sh;
+  const T *vbase = (const T *)p.v.ptr + sq.b * p.v.sb + kvh * p.v.sh;
+
+  TileLoader<D, NT, PAD> kload, vload;
+  kload.init(tid, p.k.st, p.D);
+  vload.init(tid, p.v.st, p.D);
+  // blocks whose first key lies in [0, k_full_span) hold 64 keys of the sequence
+  const uint32_t k_full_span = sq.k_len >= 64 ? (uint32_t)(sq.k_len - 64) + 1u : 0u;
+  const uint32_t k_row_bytes = (uint32_t)p.k.st * 2u, v_row_bytes = (uint32_t)p.v.st * 2u;
+  auto issue = [&](int col, int stage) {  // asynchronous copy of K/V block `col` into `stage`
+    const int key0 = col * 64;
+    char *ks = smem + stage * STAGE;
+    if ((uint32_t)key0 < k_full_span) {  // main path (one scalar compare; a padding entry is negative)
+      kload.issue_full(row_address(reinterpret_cast<const char *>(kbase), key0, k_row_bytes), ks);
+      vload.issue_full(row_address(reinterpret_cast<const char *>(vbase), key0, v_row_bytes), ks + TL::kBytes);
+      return;
+    }
+    const int valid = col < 0 ? 0 : sq.k_len - key0;
+    kload.issue(reinterpret_cast<const char *>(kbase + (int64_t)key0 * p.k.st), 0, valid, ks);
+    vload.issue(reinterpret_cast<const char *>(vbase + (int64_t)key0 * p.v.st), 0, valid, ks + TL::kBytes);
+  };
+  // operand read addresses for a tile at offset 0: row m of a 32-key half, chunk 2ks+g swizzled;
+  // transpose-read pairs of d-tile dt.  Stage, key half and k-step offsets are immediates.
+  using OA = OperandAddress<D>;
+  typename OA::type rd[KS], tr[DT][2];
+  {
+    int tro[DT][2];
+    transposed_offsets<D>(lane, tro);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) rd[ks] = OA::make(smem, TL::off(m, 2 * ks + g));
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) tr[dt][0] = OA::make(smem, tro[dt][0]), tr[dt][1] = OA::make(smem, tro[dt][1]);
+  }
+
+  floatx16 acc[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[dt][r] = 0.f;
+
+  // The union of the two rows in column order: head_a / head_b are the next unconsumed entries
+  // (scalar), pend_a / pend_b the entries after them (vector loads, first used behind a tile
+  // wait, so that no table read stalls the loop); flg_cur says which rows hold the current column.
+  constexpr int kEnd = 0x7fffffff;
+  int a_pos = e0, b_pos = emid, head_a = kEnd, head_b = kEnd, pend_a = 0, pend_b = 0;
+  int hbits_a = 0, hbits_b = 0, pbits_a = 0, pbits_b = 0;  // SUB: the entries' masks, carried like the columns
+  if (a_pos < emid) head_a = scalar_load(cols + a_pos * EW);
+  if (b_pos < e1) head_b = scalar_load(cols + b_pos * EW);
+  if (a_pos + 1 < emid) pend_a = cols[(a_pos + 1) * EW];
+  if (b_pos + 1 < e1) pend_b = cols[(b_pos + 1) * EW];
+  if constexpr (SUB) {
+    if (a_pos < emid) hbits_a = scalar_load(cols + a_pos * EW + 1);
+    if (b_pos < e1) hbits_b = scalar_load(cols + b_pos * EW + 1);
+    if (a_pos + 1 < emid) pbits_a = cols[(a_pos + 1) * EW + 1];
+    if (b_pos + 1 < e1) pbits_b = cols[(b_pos + 1) * EW + 1];
+  }
+  int col_cur = min(head_a, head_b);
+  int flg_cur = (head_a == col_cur ? 1 : 0) | (head_b == col_cur ? 2 : 0);
+  int bits_cur = ts ? hbits_b : hbits_a;  // mask of the current column in this wave's row (if it holds it)
+
+  // Q and dO fragments, lse in the log2 domain, and delta = rowsum(O * dO) - dLSE, which this
+  // kernel computes itself and also leaves in p.delta for the dK/dV pass that follows
+  wait_tile_loads();
+  __syncthreads();  // the Q and dO tiles are visible
+  vec8 qf[KS], dof[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    qf[ks] = lds_read8<vec8>(smem + ts * STAGE + TL::off(rh * 32 + m, 2 * ks + g));
+    dof[ks] = lds_read8<vec8>(smem + ts * STAGE + TL::kBytes + TL::off(rh * 32 + m, 2 * ks + g));
+  }
+#pragma unroll
+  for (int j = 0; j < OCH; ++j) {
+    const int r = tid / CPR + j * (NT / CPR), ch = tid % CPR;
+    const uint4 dow = *reinterpret_cast<const uint4 *>(smem + (r >> 6) * STAGE + TL::kBytes + TL::off(r & 63, ch));
+    float d = dot8<T>(oreg[j], dow, 0.f);
+#pragma unroll
+    for (int off = CPR / 2; off > 0; off >>= 1) d += __shfl_xor(d, off);
+    if (ch == 0) delta_rows[r] = d;
+  }
+  __syncthreads();  // the row sums are there; every wave has its fragments: both stages are free
+  if (col_cur != kEnd) issue(col_cur, 0);
+  float lse2 = INFINITY, delta = 0.f;
+  if (row_ok) {
+    lse2 = lse_raw == -INFINITY ? INFINITY : lse_raw * kLog2e;
+    delta = delta_rows[ts * 64 + rh * 32 + m] - dlse_raw;
+    if (g == 0) p.delta[((int64_t)sq.b * p.Hq + h) * p.seqs.max_q_len + qi] = delta;
+  }
+
+  auto block_step = [&](auto stage_tag) {
+    constexpr int stage = decltype(stage_tag)::value;
+    const int col = col_cur;
+    const int flg = flg_cur;
+    const int bits = bits_cur;
+    wait_tile_loads();
+    __syncthreads();  // the tile is visible; every wave is done with the other stage
+    if (flg & 1) {
+      ++a_pos;
+      head_a = a_pos < emid ? __builtin_amdgcn_readfirstlane(pend_a) : kEnd;
+      if (a_pos + 1 < emid) pend_a = cols[(a_pos + 1) * EW];
+      if constexpr (SUB) {
+        hbits_a = __builtin_amdgcn_readfirstlane(pbits_a);
+        if (a_pos + 1 < emid) pbits_a = cols[(a_pos + 1) * EW + 1];
+      }
+    }
+    if (flg & 2) {
+      ++b_pos;
+      head_b = b_pos < e1 ? __builtin_amdgcn_readfirstlane(pend_b) : kEnd;
+      if (b_pos + 1 < e1) pend_b = cols[(b_pos + 1) * EW];
+      if constexpr (SUB) {
+        hbits_b = __builtin_amdgcn_readfirstlane(pbits_b);
+        if (b_pos + 1 < e1) pbits_b = cols[(b_pos + 1) * EW + 1];
+      }
+    }
+    const int col_next = min(head_a, head_b);
+    flg_cur = (head_a == col_next ? 1 : 0) | (head_b == col_next ? 2 : 0);
+    if constexpr (SUB) bits_cur = ts ? hbits_b : hbits_a;
+    if (col_next != kEnd) issue(col_next, stage ^ 1);
+    col_cur = col_next;
+    if (!((flg >> ts) & 1)) return;  // not in this wave's row
+    if (col < 0) return;
+    constexpr int ks_ = stage * STAGE, vs_ = ks_ + TL::kBytes;  // byte offsets of this stage's K and V tiles
+
+#pragma unroll
+    for (int kh = 0; kh < 2; ++kh) {  // the two 32-key halves of the block
+      const int key0 = col * 64 + kh * 32;
+      if (key0 >= sq.k_len || (p.causal && key0 > row0 + 31)) continue;  // nothing visible (wave-uniform)
+      constexpr int kRow32 = 32 * TL::kRowBytes;
+      floatx16 s, dp;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[r] = dp[r] = 0.f;
+      // batches of operand reads, then the multiplies (the scheduler barriers keep
+      // the compiler from sinking each read next to its MFMA)
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        vec8 ka[KS / 2];
+#pragma unroll
+        for (int i = 0; i < KS / 2; ++i) ka[i] = lds_operand<vec8>(rd[half * (KS / 2) + i] + ks_ + kh * kRow32);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < KS / 2; ++i) s = M::mma(ka[i], qf[half * (KS / 2) + i], s);
+      }
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        vec8 va[KS / 2];
+#pragma unroll
+        for (int i = 0; i < KS / 2; ++i) va[i] = lds_operand<vec8>(rd[half * (KS / 2) + i] + vs_ + kh * kRow32);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < KS / 2; ++i) dp = M::mma(va[i], dof[half * (KS / 2) + i], dp);
+      }
+      // K^T operands of the dQ product do not depend on dS: fetch them now
+      vec8 kt[DT];
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) kt[dt] = lds_operand_tr<vec8>(tr[dt][0] + ks_ + kh * kRow32, tr[dt][1] + ks_ + kh * kRow32);
+
+      const bool need_mask = (key0 + 31 >= sq.k_len) || (p.causal && key0 + 31 > row0);
+      const int lim = p.causal ? min(pos, sq.k_len - 1) : sq.k_len - 1;  // last visible key of this row
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[r] = fast_exp2(fmaf(s[r], p.scale_log2, -lse2));
+      if (need_mask) {  // wave-uniform: only the diagonal block and the last, partial one pay for masks
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int key = key0 + (r >> 2) * 8 + g * 4 + (r & 3);
+          s[r] = key > lim ? 0.f : s[r];
+        }
+      }
+      if constexpr (SUB) {
+        // pattern blocks of the tile that this row does not attend: bit (row part) * f + (key part)
+        const int lb = p.csr.sub_block == 16 ? 4 : 5, f = 64 >> lb;
+        const int full = f == 4 ? 0xffff : 0xf;
+        if ((bits & full) != full) {  // wave-uniform
+          const int row_bits = bits >> (((rh * 32 + m) >> lb) * f);
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            // key kh 32 + 8 (r / 4) + 4 g + r % 4: the last two terms stay inside a part of >= 16 keys
+            const int key_part = (kh * 32 + (r >> 2) * 8) >> lb;
+            s[r] = ((row_bits >> key_part) & 1) ? s[r] : 0.f;
+          }
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[r] *= dp[r] - delta;  // dS^T without sm_scale (applied once at the end)
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        float f[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) f[i] = s[t * 8 + i];
+        const vec8 dsb = M::pack(f);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          acc[dt] = M::mma(kt[dt], dsb, acc[dt]);
+          if (t == 0)  // refill with the second k-step's operand as soon as the register is free
+            kt[dt] = lds_operand_tr<vec8>(tr[dt][0] + ks_ + kh * kRow32 + 16 * TL::kRowBytes,
+                                          tr[dt][1] + ks_ + kh * kRow32 + 16 * TL::kRowBytes);
+        }
+      }
+    }
+  };
+  while (col_cur != kEnd) {
+    block_step(IntConst<0>{});
+    if (col_cur == kEnd) break;
+    block_step(IntConst<1>{});
+  }
+
+  // every wave holds the finished dQ^T of its 32 rows
+  __syncthreads();  // the K / V stages are free: each wave stages its tile in 32 rows of them
+  {
+    const int qi0 = row0 - sq.past;  // may be negative or beyond q_len: those rows are skipped
+    T *dq_row0 = (T *)p.dq.ptr + sq.b * p.dq.sb + h * p.dq.sh + (int64_t)qi0 * p.dq.st;
+    store_tile_rows<T, D, PAD>(smem + wave * 32 * TL::kRowBytes, acc, p.sm_scale, dq_row0, p.dq.st, lane, -qi0,
+                               sq.q_len - qi0, p.D);
+  }
+}
+
+// ---------------------------------------------------------------------------
 // dK / dV pass
 // ---------------------------------------------------------------------------
 // One workgroup = one 64-key column block of one kv head, 4 waves, two workgroups per CU (the
@@ -554,6 +861,22 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 
       }
     };
 
+    // The column's entries live in the lanes of a register (lane l: entry l of the current chunk of
+    // 64) and are picked out with a lane read: a scalar load per block, waited for on the spot,
+    // cost the pass 13 % (every wave of the workgroup stood at the barrier behind it).  The one
+    // vector load per chunk is waited for before any tile request of the head is in flight.
+    const int nblk = e1 - e0;
+    int my_rows = lane < nblk ? rows[lane * EW] : -1;
+    int my_bits = 0;
+    if constexpr (SUB) my_bits = lane < nblk ? rows[lane * EW + 1] : 0;
+    auto entry_row = [&](int k) {  // q block of entry k; called with k ascending
+      if (k > 0 && (k & 63) == 0) {  // (columns of more than 64 entries: next chunk; the wait also covers the tiles in flight)
+        my_rows = k + lane < nblk ? rows[(k + lane) * EW] : -1;
+        if constexpr (SUB) my_bits = k + lane < nblk ? rows[(k + lane) * EW + 1] : 0;
+      }
+      return __builtin_amdgcn_readlane(my_rows, k & 63);
+    };
+
     // The loop is instantiated once per role (not branched inside), so that the accumulators
     // are not merged through a join every iteration.
     auto run_head = [&](auto role_tag) {
@@ -562,8 +885,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 
     bool exact = true;                // every wave has issued exactly LPT load instructions per outstanding step
     static_assert(S::kAhead == 2, "the first block's two steps are requested together");
     int rb_next = 0;                  // q block of the next step to request (steps 2k and 2k + 1 share block k)
+    int rb_cur = 0, bits_nxt = 0;     // q block of the step being worked on; SUB: mask of the block after it
     if (nstep > 0) {
-      rb_next = scalar_load(rows);
+      rb_next = entry_row(0);
+      rb_cur = rb_next;
+      if constexpr (SUB) bits_nxt = __builtin_amdgcn_readlane(my_bits, 0);
       for (int i = 0; i < S::kAhead; ++i, ++issued) {
         exact = issue(rb_next, i, iq, ido) && exact;
         iq = iq + 1 == S::kQStages ? 0 : iq + 1;
@@ -589,8 +915,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 
       const int half = t & 1;
       wait_tiles_ahead<LPT>(exact ? issued - t - 1 : 0);
       __syncthreads();  // step t is visible, so is P of step t - 1; the stages of step t - 2 are free
+      // (requests run exactly one block ahead of the work: at an even step the block that was
+      // requested last becomes the current one)
+      if (half == 0 && t > 0) rb_cur = rb_next;
+      if constexpr (SUB) {
+        if (half == 0) bits = bits_nxt;
+      }
       if (issued < nstep) {
-        if ((issued & 1) == 0) rb_next = scalar_load(rows + (issued >> 1) * EW);
+        if ((issued & 1) == 0) {
+          rb_next = entry_row(issued >> 1);
+          if constexpr (SUB) bits_nxt = __builtin_amdgcn_readlane(my_bits, (issued >> 1) & 63);
+        }
         exact = issue(rb_next, issued & 1, iq, ido) && exact;
         iq = iq + 1 == S::kQStages ? 0 : iq + 1;
         ido = ido + 1 == S::kDoStages ? 0 : ido + 1;
@@ -598,12 +933,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 
       }
       const char *qs_ = smem + S::kQ + cq * S::kTile, *dos_ = smem + S::kDo + cdo * S::kTile;
       if constexpr (!kDp) {
-        if (half == 0) {
-          if constexpr (SUB)
-            scalar_load2(rows + (t >> 1) * EW, rows + (t >> 1) * EW + 1, rbq, bits);
-          else
-            rbq = scalar_load(rows + (t >> 1));
-        }
+        rbq = rb_cur;
         const int pos0 = rbq * 64 + half * 32;  // first q position of this step
         const float *lse_s = reinterpret_cast<const float *>(smem + S::kVec + cq * 256);
         // S = Q K^T : rows = 32 q positions, cols = 32 keys
@@ -761,22 +1091,22 @@ template __global__ void mfma_dkdv_kernel<bf16_t, 256, true, false>(const BwdPar
 template __global__ void mfma_dkdv_kernel<bf16_t, 256, true, true>(const BwdParams, int);
 template __global__ void mfma_dkdv_kernel<f16_t, 256, true, false>(const BwdParams, int);
 template __global__ void mfma_dkdv_kernel<f16_t, 256, true, true>(const BwdParams, int);
-template __global__ void mfma_dq_kernel<bf16_t, 128, false, false>(const BwdParams, int);
-template __global__ void mfma_dq_kernel<bf16_t, 128, true, false>(const BwdParams, int);
-template __global__ void mfma_dq_kernel<bf16_t, 128, false, true>(const BwdParams, int);
-template __global__ void mfma_dq_kernel<bf16_t, 128, true, true>(const BwdParams, int);
-template __global__ void mfma_dq_kernel<bf16_t, 64, false, false>(const BwdParams, int);
-template __global__ void mfma_dq_kernel<bf16_t, 64, true, false>(const BwdParams, int);
-template __global__ void mfma_dq_kernel<bf16_t, 64, false, true>(const BwdParams, int);
-template __global__ void mfma_dq_kernel<bf16_t, 64, true, true>(const BwdParams, int);
-template __global__ void mfma_dq_kernel<f16_t, 128, false, false>(const BwdParams, int);
-template __global__ void mfma_dq_kernel<f16_t, 128, true, false>(const BwdParams, int);
-template __global__ void mfma_dq_kernel<f16_t, 128, false, true>(const BwdParams, int);
-template __global__ void mfma_dq_kernel<f16_t, 128, true, true>(const BwdParams, int);
-template __global__ void mfma_dq_kernel<f16_t, 64, false, false>(const BwdParams, int);
-template __global__ void mfma_dq_kernel<f16_t, 64, true, false>(const BwdParams, int);
-template __global__ void mfma_dq_kernel<f16_t, 64, false, true>(const BwdParams, int);
-template __global__ void mfma_dq_kernel<f16_t, 64, true, true>(const BwdParams, int);
+template __global__ void mfma_dq_pair_kernel<bf16_t, 128, false, false>(const BwdParams, int);
+template __global__ void mfma_dq_pair_kernel<bf16_t, 128, true, false>(const BwdParams, int);
+template __global__ void mfma_dq_pair_kernel<bf16_t, 128, false, true>(const BwdParams, int);
+template __global__ void mfma_dq_pair_kernel<bf16_t, 128, true, true>(const BwdParams, int);
+template __global__ void mfma_dq_pair_kernel<bf16_t, 64, false, false>(const BwdParams, int);
+template __global__ void mfma_dq_pair_kernel<bf16_t, 64, true, false>(const BwdParams, int);
+template __global__ void mfma_dq_pair_kernel<bf16_t, 64, false, true>(const BwdParams, int);
+template __global__ void mfma_dq_pair_kernel<bf16_t, 64, true, true>(const BwdParams, int);
+template __global__ void mfma_dq_pair_kernel<f16_t, 128, false, false>(const BwdParams, int);
+template __global__ void mfma_dq_pair_kernel<f16_t, 128, true, false>(const BwdParams, int);
+template __global__ void mfma_dq_pair_kernel<f16_t, 128, false, true>(const BwdParams, int);
+template __global__ void mfma_dq_pair_kernel<f16_t, 128, true, true>(const BwdParams, int);
+template __global__ void mfma_dq_pair_kernel<f16_t, 64, false, false>(const BwdParams, int);
+template __global__ void mfma_dq_pair_kernel<f16_t, 64, true, false>(const BwdParams, int);
+template __global__ void mfma_dq_pair_kernel<f16_t, 64, false, true>(const BwdParams, int);
+template __global__ void mfma_dq_pair_kernel<f16_t, 64, true, true>(const BwdParams, int);
 template __global__ void mfma_dkdv_kernel<bf16_t, 128, false, false>(const BwdParams, int);
 template __global__ void mfma_dkdv_kernel<bf16_t, 128, true, false>(const BwdParams, int);
 template __global__ void mfma_dkdv_kernel<bf16_t, 128, false, true>(const BwdParams, int);
@@ -851,15 +1181,22 @@ static int launch_bwd_td(const BwdParams &p, void *workspace, size_t workspace_b
   const SeqView &s = p.seqs;
   constexpr int smem_dq = 2 * 2 * Tile<D>::kBytes;
   constexpr int smem_dkdv = DkdvSmem<D>::kBytes;
-  DK_ALLOW_DYNAMIC_LDS((mfma_dq_kernel<T, D, PAD, SUB>), smem_dq);
   DK_ALLOW_DYNAMIC_LDS((mfma_dkdv_kernel<T, D, PAD, SUB>), smem_dkdv);
   const int past = p.causal ? s.max_k_len - s.max_q_len : 0;
   const int tiles = (past + s.max_q_len - 1) / 64 - past / 64 + 1;
   const int cblocks = cdiv(s.max_k_len, 64);
   DK_REQUIRE(tiles <= 65535 && cblocks <= 65535, "sequence too long for one launch");
   // dQ first: it also writes delta, which the dK/dV pass reads
-  DK_NOTE_KERNEL("mfma_dq_kernel");
-  hipLaunchKernelGGL((mfma_dq_kernel<T, D, PAD, SUB>), dim3(p.Hq, tiles, s.batch), dim3(256), smem_dq, stream, p, tiles);
+  if constexpr (D <= 128) {  // two table rows per workgroup
+    const int pairs = (((past + s.max_q_len - 1) / 64) >> 1) - ((past / 64) >> 1) + 1;
+    DK_ALLOW_DYNAMIC_LDS((mfma_dq_pair_kernel<T, D, PAD, SUB>), smem_dq);
+    DK_NOTE_KERNEL("mfma_dq_pair_kernel");
+    hipLaunchKernelGGL((mfma_dq_pair_kernel<T, D, PAD, SUB>), dim3(p.Hq, pairs, s.batch), dim3(256), smem_dq, stream, p, pairs);
+  } else {
+    DK_ALLOW_DYNAMIC_LDS((mfma_dq_kernel<T, D, PAD, SUB>), smem_dq);
+    DK_NOTE_KERNEL("mfma_dq_kernel");
+    hipLaunchKernelGGL((mfma_dq_kernel<T, D, PAD, SUB>), dim3(p.Hq, tiles, s.batch), dim3(256), smem_dq, stream, p, tiles);
+  }
   DK_HIP_CHECK(hipGetLastError());
   // With several q heads per kv head a workgroup per kv head walks all of them, and the longest
   // column (a vertical one near the start: every later q block, times the group size) alone

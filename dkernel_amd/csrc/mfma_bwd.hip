@@ -861,22 +861,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 
       }
     };
 
-    // The column's entries live in the lanes of a register (lane l: entry l of the current chunk of
-    // 64) and are picked out with a lane read: a scalar load per block, waited for on the spot,
-    // cost the pass 13 % (every wave of the workgroup stood at the barrier behind it).  The one
-    // vector load per chunk is waited for before any tile request of the head is in flight.
-    const int nblk = e1 - e0;
-    int my_rows = lane < nblk ? rows[lane * EW] : -1;
-    int my_bits = 0;
-    if constexpr (SUB) my_bits = lane < nblk ? rows[lane * EW + 1] : 0;
-    auto entry_row = [&](int k) {  // q block of entry k; called with k ascending
-      if (k > 0 && (k & 63) == 0) {  // (columns of more than 64 entries: next chunk; the wait also covers the tiles in flight)
-        my_rows = k + lane < nblk ? rows[(k + lane) * EW] : -1;
-        if constexpr (SUB) my_bits = k + lane < nblk ? rows[(k + lane) * EW + 1] : 0;
-      }
-      return __builtin_amdgcn_readlane(my_rows, k & 63);
-    };
-
     // The loop is instantiated once per role (not branched inside), so that the accumulators
     // are not merged through a join every iteration.
     auto run_head = [&](auto role_tag) {
@@ -885,11 +869,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 
     bool exact = true;                // every wave has issued exactly LPT load instructions per outstanding step
     static_assert(S::kAhead == 2, "the first block's two steps are requested together");
     int rb_next = 0;                  // q block of the next step to request (steps 2k and 2k + 1 share block k)
-    int rb_cur = 0, bits_nxt = 0;     // q block of the step being worked on; SUB: mask of the block after it
     if (nstep > 0) {
-      rb_next = entry_row(0);
-      rb_cur = rb_next;
-      if constexpr (SUB) bits_nxt = __builtin_amdgcn_readlane(my_bits, 0);
+      rb_next = scalar_load(rows);
       for (int i = 0; i < S::kAhead; ++i, ++issued) {
         exact = issue(rb_next, i, iq, ido) && exact;
         iq = iq + 1 == S::kQStages ? 0 : iq + 1;
@@ -915,17 +896,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 
       const int half = t & 1;
       wait_tiles_ahead<LPT>(exact ? issued - t - 1 : 0);
       __syncthreads();  // step t is visible, so is P of step t - 1; the stages of step t - 2 are free
-      // (requests run exactly one block ahead of the work: at an even step the block that was
-      // requested last becomes the current one)
-      if (half == 0 && t > 0) rb_cur = rb_next;
-      if constexpr (SUB) {
-        if (half == 0) bits = bits_nxt;
-      }
       if (issued < nstep) {
-        if ((issued & 1) == 0) {
-          rb_next = entry_row(issued >> 1);
-          if constexpr (SUB) bits_nxt = __builtin_amdgcn_readlane(my_bits, (issued >> 1) & 63);
-        }
+        if ((issued & 1) == 0) rb_next = scalar_load(rows + (issued >> 1) * EW);
         exact = issue(rb_next, issued & 1, iq, ido) && exact;
         iq = iq + 1 == S::kQStages ? 0 : iq + 1;
         ido = ido + 1 == S::kDoStages ? 0 : ido + 1;
@@ -933,7 +905,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 
       }
       const char *qs_ = smem + S::kQ + cq * S::kTile, *dos_ = smem + S::kDo + cdo * S::kTile;
       if constexpr (!kDp) {
-        rbq = rb_cur;
+        if (half == 0) {
+          if constexpr (SUB)
+            scalar_load2(rows + (t >> 1) * EW, rows + (t >> 1) * EW + 1, rbq, bits);
+          else
+            rbq = scalar_load(rows + (t >> 1));
+        }
         const int pos0 = rbq * 64 + half * 32;  // first q position of this step
         const float *lse_s = reinterpret_cast<const float *>(smem + S::kVec + cq * 256);
         // S = Q K^T : rows = 32 q positions, cols = 32 keys

@@ -17,6 +17,10 @@ size_t mfma_fwd_workspace_bytes(const FwdParams &p);
 bool mfma_bwd_supported(const BwdParams &p, int dtype);
 int launch_mfma_bwd(const BwdParams &p, int dtype, void *workspace, size_t workspace_bytes, hipStream_t stream);
 size_t mfma_bwd_workspace_bytes(const BwdParams &p);
+bool mfma_f32_fwd_supported(const FwdParams &p, int dtype);
+bool mfma_f32_bwd_supported(const BwdParams &p, int dtype);
+int launch_mfma_f32_fwd(const FwdParams &p, hipStream_t stream);
+int launch_mfma_f32_bwd(const BwdParams &p, hipStream_t stream);
 bool decode_supported(const FwdParams &p, int dtype);
 size_t decode_workspace_bytes(const FwdParams &p);
 int launch_decode(const FwdParams &p, int dtype, void *workspace, size_t workspace_bytes, hipStream_t stream);
@@ -227,6 +231,7 @@ int dk_fwd(const dk_fwd_args *a) {
       return launch_decode(p, a->dtype, a->workspace, a->workspace_bytes, stream);
     if (mfma_fwd_supported(p, a->dtype))
       return launch_mfma_fwd(p, a->dtype, a->workspace, a->workspace_bytes, stream);
+    if (mfma_f32_fwd_supported(p, a->dtype)) return launch_mfma_f32_fwd(p, stream);
     if (a->impl == DK_IMPL_MFMA)
       return fail(DK_ERR_UNSUPPORTED, "no MFMA forward kernel for dtype %d, head_dim %d, tiles (%d, %d)", a->dtype,
                   p.D, p.csr.block_rows, p.csr.block_cols);
@@ -292,6 +297,7 @@ int dk_bwd(const dk_bwd_args *a) {
     if (mfma_bwd_supported(p, a->dtype)) {
       return launch_mfma_bwd(p, a->dtype, a->workspace, a->workspace_bytes, stream);
     }
+    if (mfma_f32_bwd_supported(p, a->dtype)) return launch_mfma_f32_bwd(p, stream);
     if (a->impl == DK_IMPL_MFMA)
       return fail(DK_ERR_UNSUPPORTED, "no MFMA backward kernel for dtype %d, head_dim %d, tiles (%d, %d)",
                   a->dtype, p.D, p.csr.block_rows, p.csr.block_cols);

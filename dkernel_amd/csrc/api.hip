@@ -280,7 +280,7 @@ int dk_fwd_paged(const dk_fwd_args *a, const dk_paged_kv *pg) {
   if (a->impl == DK_IMPL_GENERIC || !decode_supported(p, a->dtype))
     return fail(DK_ERR_UNSUPPORTED,
                 "paged K/V is served by the split-KV decode kernels only (one query token per sequence, 16-bit "
-                "floats, head_dim a multiple of 8 up to 128, 64 x 64 tiles, causal)");
+                "floats, head_dim a multiple of 8 up to 256, 64 x 64 tiles, causal)");
   DK_REQUIRE(a->workspace && a->workspace_bytes >= decode_workspace_bytes(p), "decode workspace too small");
   return launch_decode(p, a->dtype, a->workspace, a->workspace_bytes, (hipStream_t)a->stream);
 }

@@ -1,6 +1,6 @@
 // Split-KV decode kernels for gfx950: one new query token per sequence over
 // padded (left or right), unpadded, packed or paged K/V, bf16 / fp16 (paged
-// pools also fp8), head_dim a multiple of 8 up to 128, 64 x 64 tiles,
+// pools also fp8), head_dim a multiple of 8 up to 256, 64 x 64 tiles,
 // grouped-query attention with all q heads of a kv head sharing the
 // look-up-table row.  The step is HBM-bound (every attended K/V byte is read
 // exactly once, for all q heads of the group together), so the design goal is
@@ -25,7 +25,8 @@
 // A wave works on half blocks (32 keys): 2 x 8.5 KB of private LDS tiles and
 // the next half block prefetched into registers, so 8 waves are resident per
 // CU (2 per SIMD, <= 256 VGPRs each): one wave's loads overlap the other's
-// multiplies on the same SIMD.
+// multiplies on the same SIMD.  (Head dims above 128: 256-wide tiles, 2 x 33 KB per wave, one
+// workgroup of four waves per CU and one wave per SIMD.)
 #include <algorithm>
 #include <type_traits>
 
@@ -102,7 +103,7 @@ __device__ __forceinline__ uint4 fp8x8_to(uint2 w) {
 // workgroup is finished here (the waves exchange their partials through LDS and write O / LSE);
 // longer rows leave their partials in the workspace for decode_combine_kernel.
 template <typename T, int D, bool PAD, bool SUB, bool PAGED, bool KV8, int W>
-__global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(2, 2))) void decode_partial_kernel(
+__global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(D == 256 ? 1 : 2, D == 256 ? 1 : 2))) void decode_partial_kernel(
     const FwdParams p, float *ws, int unit_blocks, int max_units) {
   using M = Mma<T>;
   using vec8 = typename M::vec8;
@@ -506,7 +507,9 @@ bool decode_supported(const FwdParams &p, int dtype) {
   const int ratio = p.Hq / p.Hkv;
   const bool shared_row = p.csr.num_heads == 1 || (p.csr.num_heads == p.Hkv && p.Hkv != p.Hq) || ratio == 1 ||
                           (p.csr.num_heads == p.Hq && p.csr.group % ratio == 0);
-  return (dtype == DK_BF16 || dtype == DK_F16) && mfma_head_dim_ok(p.D) && p.D <= 128 && p.csr.block_rows == 64 &&
+  const int width = mfma_tile_width(p.D);
+  const int lds = kDecodeWaves * (2 * 32 * (width * 2 + 16) + ratio * width * 2);  // DecSmem<width>::wave_bytes
+  return (dtype == DK_BF16 || dtype == DK_F16) && mfma_head_dim_ok(p.D) && lds <= 160 * 1024 && p.csr.block_rows == 64 &&
          p.csr.block_cols == 64 && p.vec_ok &&
          (p.csr.entry_width == 1 || p.csr.sub_block != 0) &&
          (p.seqs.packed ? (p.seqs.packed & 2) != 0 : p.seqs.max_q_len == 1) && ratio <= 32 && shared_row && p.causal;
@@ -539,6 +542,9 @@ static int launch_decode_td(const FwdParams &p, float *ws, hipStream_t stream) {
 
 template <typename T, bool PAGED>
 static int launch_decode_tp(const FwdParams &p, float *ws, hipStream_t stream) {
+  if (p.D > 128)  // 256-wide tiles (always the zero-padding instantiation), one wave per SIMD
+    return p.csr.sub_block ? launch_decode_td<T, 256, true, true, PAGED>(p, ws, stream)
+                           : launch_decode_td<T, 256, true, false, PAGED>(p, ws, stream);
   if (p.csr.sub_block) {  // entries carry a bit mask over the pattern's 16- or 32-token blocks
     if (p.D == 128) return launch_decode_td<T, 128, false, true, PAGED>(p, ws, stream);
     if (p.D == 64) return launch_decode_td<T, 64, false, true, PAGED>(p, ws, stream);

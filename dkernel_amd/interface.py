@@ -304,7 +304,7 @@ class SparseAttention(torch.nn.Module):
         sequence); context_lens: int32 (batch,) keys per sequence including the new token's.
         Pools of dtype torch.float8_e4m3fn hold K / k_scale and V / v_scale (head_dim 64 / 128,
         blocks of at least 64).  Needs the matrix-core decode kernels (bf16 / fp16, head_dim a multiple
-        of 8 up to 128).  No counterpart in the reference."""
+        of 8 up to 256).  No counterpart in the reference."""
         from .ops import paged_decode_attn
         assert self.kwargs.get('causal', True), "paged decode is causal"
         if self.kernel_tile is not None:

@@ -8,7 +8,7 @@ import pytest
 import torch
 
 from dkernel_amd import LocalStrideSparseAttention, SparseAttention, combine_attn_partitions, get_sparse_attn_mask
-from dkernel_amd import ops
+from dkernel_amd import _lib, ops
 from oracle import attention as OA
 from oracle import layout as OL
 from helpers import F32_TOL, LSE_TOL, TOL, assert_close, expand_heads, make_qkv, oracle_fwd
@@ -309,6 +309,13 @@ def test_decode_head_dims_below_tile_width(impl, D, left):
     _decode_case(64, None, left, D)
 
 
+@pytest.mark.parametrize("D,bs,left", [(256, 64, True), (192, 64, False), (160, 32, True), (136, 128, False)])
+def test_decode_head_dims_above_128(D, bs, left):
+    """Head dims above 128 take the split-KV decode kernels too (256-wide tiles)."""
+    _decode_case(bs, None, left, D)
+    assert _lib.lib().dk_last_kernels().decode().startswith("decode_partial_kernel [T = dk::bf16_t, D = 256")
+
+
 @pytest.mark.parametrize("bs,D,left", [(16, 96, True), (32, 40, False)])
 def test_decode_small_blocks_with_padded_head_dims(bs, D, left):
     """Blocks of 16 / 32 (masked tiles) and a head dim below the tile width, matrix-core kernels forced."""
@@ -322,7 +329,8 @@ def test_decode_small_blocks_with_padded_head_dims(bs, D, left):
 @pytest.mark.parametrize("page_size,bs,D,head_major", [(16, 64, 128, False), (32, 64, 128, True), (64, 64, 96, False),
                                                         (128, 64, 128, False), (16, 16, 128, False),
                                                         (32, 128, 64, True), (256, 32, 128, False),
-                                                        (16, 16, 96, False), (64, 32, 40, True)])
+                                                        (16, 16, 96, False), (64, 32, 40, True),
+                                                        (16, 64, 256, False), (64, 32, 192, True)])
 def test_paged_decode(page_size, bs, D, head_major):
     """Single-token decode over a paged K/V cache: pages scattered in the pools, table rows padded
     with -1 past each sequence, pools token-major or head-major inside a page; against the oracle

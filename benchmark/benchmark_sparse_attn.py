@@ -1,12 +1,15 @@
 """Latency sweep of the block-sparse attention over sequence length and vertical stride.
 
     python benchmark/benchmark_sparse_attn.py [--mode fwd|bwd|both] [--max-log2 16] [--csv out.csv]
+        [--batch 4 --heads 16 --head-dim 128 --local-tokens 512 --dtype bfloat16 --impl auto]
 
 Same sweep as the reference's benchmark/benchmark_sparse_attn.py (its defaults at
 lines 24-40 and 67: batch 4, 16 heads, head_dim 128, local window 512 tokens, block 64,
 bf16, sequence lengths 2^10 .. 2^16, vert_stride in {1, 4, 16}, warm-up 25 / 100 timed
 repetitions), next to PyTorch's dense causal scaled_dot_product_attention when that runs on
-the box.  Prints one table per mode (milliseconds) and optionally writes a CSV.
+the box.  Prints one table per mode (milliseconds) and optionally writes a CSV.  The shape, the
+dtype and the kernel family (`--impl generic` = the fp32-FMA kernels, `mfma` = matrix cores only)
+can be changed, e.g. for fp32 on the matrix cores against the generic kernels.
 """
 import argparse
 import csv
@@ -17,9 +20,10 @@ import sys
 import torch
 
 sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
-from dkernel_amd import LocalStrideSparseAttention  # noqa: E402
+from dkernel_amd import LocalStrideSparseAttention, ops  # noqa: E402
 
 B, H, D, BLOCK, LOCAL_TOKENS = 4, 16, 128, 64, 512
+DTYPE = torch.bfloat16
 
 
 def timeit(fn, warmup, reps):
@@ -38,7 +42,7 @@ def timeit(fn, warmup, reps):
 def bench_one(L, vert, mode, warmup, reps):
     dev = "cuda:0"
     g = torch.Generator(device=dev).manual_seed(20)
-    q, k, v, do = (torch.randn(B, L, H, D, generator=g, device=dev, dtype=torch.bfloat16) for _ in range(4))
+    q, k, v, do = (torch.randn(B, L, H, D, generator=g, device=dev, dtype=DTYPE) for _ in range(4))
     sm = 1.0 / math.sqrt(D)
     mod = LocalStrideSparseAttention(H, L, BLOCK, LOCAL_TOKENS // BLOCK, vert).to(dev)
     nnz = int(mod.layout_csr_crow[:, -1].sum().item())
@@ -57,7 +61,7 @@ def bench_one(L, vert, mode, warmup, reps):
 def bench_dense(L, mode, warmup, reps):
     dev = "cuda:0"
     g = torch.Generator(device=dev).manual_seed(20)
-    q, k, v, do = (torch.randn(B, H, L, D, generator=g, device=dev, dtype=torch.bfloat16) for _ in range(4))
+    q, k, v, do = (torch.randn(B, H, L, D, generator=g, device=dev, dtype=DTYPE) for _ in range(4))
     f = torch.nn.functional.scaled_dot_product_attention
     if mode == "fwd":
         with torch.no_grad():
@@ -69,6 +73,8 @@ def bench_dense(L, mode, warmup, reps):
 
 
 def main():
+    global B, H, D, LOCAL_TOKENS, DTYPE
+    defaults = (B, H, D, LOCAL_TOKENS)
     ap = argparse.ArgumentParser()
     ap.add_argument("--mode", default="both", choices=["fwd", "bwd", "both"])
     ap.add_argument("--min-log2", type=int, default=10)
@@ -78,11 +84,20 @@ def main():
     ap.add_argument("--reps", type=int, default=100)
     ap.add_argument("--no-dense", action="store_true")
     ap.add_argument("--csv", default=None)
+    ap.add_argument("--batch", type=int, default=defaults[0])
+    ap.add_argument("--heads", type=int, default=defaults[1])
+    ap.add_argument("--head-dim", type=int, default=defaults[2])
+    ap.add_argument("--local-tokens", type=int, default=defaults[3])
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float16", "float32"])
+    ap.add_argument("--impl", default="auto", choices=["auto", "generic", "mfma"])
     args = ap.parse_args()
+    B, H, D, LOCAL_TOKENS, DTYPE = args.batch, args.heads, args.head_dim, args.local_tokens, getattr(torch, args.dtype)
+    ops.set_impl(args.impl)
     verts = [int(x) for x in args.verts.split(",")]
     rows = []
     for mode in (["fwd", "bwd"] if args.mode == "both" else [args.mode]):
-        print(f"== {mode}: b={B} h={H} d={D} bf16, block {BLOCK}, local {LOCAL_TOKENS} tokens; ms (effective TFLOP/s)")
+        print(f"== {mode}: b={B} h={H} d={D} {args.dtype}, block {BLOCK}, local {LOCAL_TOKENS} tokens, kernels: {args.impl}; "
+              "ms (effective TFLOP/s)")
         print("seqlen".rjust(8) + "".join(f"vert={v}".rjust(22) for v in verts) + "dense sdpa".rjust(14))
         for lg in range(args.min_log2, args.max_log2 + 1):
             L = 1 << lg

@@ -350,7 +350,9 @@ def test_c_abi_argument_checks_fail_before_any_launch():
     assert need > 0 and need % (2 * 8 * 130 * 4) == 0 and need // (2 * 8 * 130 * 4) >= 4
     a.seqs.max_q_len = 7                       # neither decode nor prefill of the same length
     assert lib.dk_fwd_workspace_bytes(ctypes.byref(a)) == 0
-    a = _fake_fwd_args(D=160)                  # no matrix-core decode kernel for this head_dim
+    a = _fake_fwd_args(D=160)                  # head dims above 128 decode on 256-wide tiles
+    assert lib.dk_fwd_workspace_bytes(ctypes.byref(a)) > 0
+    a = _fake_fwd_args(D=164)                  # not a multiple of 8: no matrix-core decode kernel
     assert lib.dk_fwd_workspace_bytes(ctypes.byref(a)) == 0
 
     # backward: paddings are refused as in the reference; GQA asks for fp32 per-head partials

@@ -1,6 +1,6 @@
 """Shader clock and board power while a kernel runs back to back for a few seconds: the headline
-sparse forward and a plain bf16 GEMM of the vendor library (torch.matmul, 8192^3), each on random
-and on all-zero operands.  Shows how far below the 2.4 GHz of the datasheet peak the part clocks
+sparse forward a plain bf16 GEMM of the vendor library (torch.matmul, 8192^3) and the forward + backward
+benchmark workload, each on random and on all-zero operands.  Shows how far below the 2.4 GHz of the datasheet peak the part clocks
 under matrix-core load with real data, and what rate the vendor's own GEMM sustains then.
 
     python benchmark/probe_clocks.py            (needs rocm-smi on PATH; reads, changes nothing)
@@ -92,6 +92,21 @@ def main():
         az, bz = torch.zeros_like(a), torch.zeros_like(b)
         measure("vendor GEMM 8192^3 bf16, zeros", lambda: torch.matmul(az, bz), gemm_flop)
         measure("sparse forward (headline), random data, again", lambda: mod(q, k, v, sm, return_lse=True), fwd_flop)
+    # backward workload of bench.py: one batch entry, 32 heads (MHA); forward + backward per call, so the rate
+    # quoted is that of the 3.5 x forward work (2 + 5 of the products counted)
+    modb = LocalStrideSparseAttention(32, L, 64, 16, 8).to(DEV)
+    for zeros in (False, True):
+        qb, kb, vb, do = (torch.randn(1, L, 32, D, generator=g).to(torch.bfloat16).to(DEV) for _ in range(4))
+        if zeros:
+            qb, kb, vb, do = (torch.zeros_like(x) for x in (qb, kb, vb, do))
+        qb, kb, vb = (x.requires_grad_() for x in (qb, kb, vb))
+
+        def step():
+            out = modb(qb, kb, vb, sm)
+            out.backward(do)
+            qb.grad = kb.grad = vb.grad = None
+
+        measure(f"sparse forward + backward (MHA), {'zeros' if zeros else 'random data'}", step, 3.5 * 4.0 * 64 * 64 * D * 87008)
 
 
 if __name__ == "__main__":

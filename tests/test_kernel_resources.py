@@ -4,7 +4,8 @@ Every instantiation of the MFMA kernels must stay free of scratch memory: next t
 asynchronous HBM -> LDS tile copies a scratch reload waits for every copy in flight, and a
 change that is neutral on the benchmark shapes has pushed other head dims into spills before
 (forward 0.28 -> 0.78 ms at head_dim 192).  hipcc reports the usage of each kernel with
--Rpass-analysis=kernel-resource-usage; the three files are compiled in parallel.
+-Rpass-analysis=kernel-resource-usage; the files are compiled in parallel, each with the extra
+flags the Makefile gives it (EXTRA_<file> lines).
 """
 from __future__ import annotations
 
@@ -25,8 +26,15 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xclang", "-tar
 ALLOWED = re.compile(r"mfma_fwd_kernelI\w+Li256ELi1E")
 
 
+def _extra_flags(src):
+    stem = os.path.splitext(src)[0]
+    with open(os.path.join(CSRC, "Makefile")) as f:
+        m = re.search(rf"^EXTRA_{stem}\s*:=\s*(.*)$", f.read(), re.M)
+    return m.group(1).split() if m else []
+
+
 def _usage(src, tmp):
-    out = subprocess.run([HIPCC, *FLAGS, os.path.join(CSRC, src), "-o", os.path.join(tmp, src + ".o")],
+    out = subprocess.run([HIPCC, *FLAGS, *_extra_flags(src), os.path.join(CSRC, src), "-o", os.path.join(tmp, src + ".o")],
                          capture_output=True, text=True, cwd=CSRC)
     assert out.returncode == 0, out.stderr[-2000:]
     usage, name = {}, None
@@ -42,8 +50,10 @@ def _usage(src, tmp):
 
 @pytest.mark.skipif(shutil.which(HIPCC) is None, reason="hipcc not installed")
 def test_mfma_kernels_use_no_scratch(tmp_path):
-    with concurrent.futures.ThreadPoolExecutor(3) as pool:
-        results = list(pool.map(lambda s: _usage(s, str(tmp_path)), ["mfma_fwd.hip", "mfma_bwd.hip", "decode.hip"]))
+    assert _extra_flags("mfma_fwd.hip"), "per-file flags of the Makefile not found"
+    with concurrent.futures.ThreadPoolExecutor(4) as pool:
+        results = list(pool.map(lambda s: _usage(s, str(tmp_path)),
+                                ["mfma_fwd.hip", "mfma_bwd.hip", "decode.hip", "mfma_f32.hip"]))
     usage = {k: v for r in results for k, v in r.items()}
     assert len(usage) > 100, "kernel resource remarks not found"
     spilling = {k: v for k, v in usage.items() if v and not ALLOWED.search(k)}

@@ -319,6 +319,18 @@ def main():
                            "roofline": roofline("hbm", byts, ed, dec_traffic, byts),
                            "roofline_eager_events": roofline("hbm", byts, ed_eager, dec_traffic, byts)}
         extra["decode"]["kernel_us"] = extra["decode"]["graph_step_us"]   # former name of the same figure
+        del kv_sets
+        # ---- merge of two K/V partitions (combine_attn_partitions) at the packed configuration's size ----
+        from dkernel_amd import combine_attn_partitions
+        Tc, Hc = 16384, 16
+        parts = [(gen((Tc, Hc, D), g, torch.bfloat16).to(dev), gen((Hc, Tc), g, torch.float32).to(dev)) for _ in range(2)]
+        with torch.no_grad():
+            _, ec, _ = time_steps(lambda: combine_attn_partitions(*parts), max(10, args.steps), 3)
+        # two outputs read, one written (bf16), two log-sum-exps read (fp32)
+        comb_bytes = 3 * Tc * Hc * D * 2 + 2 * Tc * Hc * 4
+        extra["combine"] = {"workload": "2 partitions of packed (16384 tokens, 16 heads, d=128) bf16 outputs + fp32 LSE",
+                            "us": round(ec * 1e3, 2), "kernels": lib.dk_last_kernels().decode(),
+                            "roofline": roofline("hbm", comb_bytes, ec, (None, "not profiled"), comb_bytes)}
         out["extra"] = extra
 
     if not args.no_cpu:

@@ -63,6 +63,15 @@ class PagedKV(C.Structure):
                 ("page_size", i32), ("kv_dtype", i32), ("k_scale", f32), ("v_scale", f32)]
 
 
+MAX_PARTITIONS = 8  # DK_MAX_PARTITIONS
+
+
+class CombineArgs(C.Structure):
+    _fields_ = [("num_partitions", i32), ("dtype", i32), ("n0", i32), ("n1", i32), ("n2", i32), ("head_dim", i32),
+                ("out", Tensor), ("dout", Tensor), ("parts", Tensor * MAX_PARTITIONS), ("lses", RowVec * MAX_PARTITIONS),
+                ("dparts", Tensor * MAX_PARTITIONS), ("dlses", RowVec * MAX_PARTITIONS), ("stream", vp)]
+
+
 # name -> (restype, argtypes); every symbol include/dkernel_hip.h declares
 SYMBOLS = {
     "dk_version": (C.c_int, []),
@@ -80,6 +89,8 @@ SYMBOLS = {
     "dk_fwd_paged": (C.c_int, [C.POINTER(FwdArgs), C.POINTER(PagedKV)]),
     "dk_bwd": (C.c_int, [C.POINTER(BwdArgs)]),
     "dk_bwd_workspace_bytes": (C.c_size_t, [C.POINTER(BwdArgs)]),
+    "dk_combine": (C.c_int, [C.POINTER(CombineArgs)]),
+    "dk_combine_bwd": (C.c_int, [C.POINTER(CombineArgs)]),
 }
 
 _lib = None

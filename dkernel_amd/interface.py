@@ -14,6 +14,7 @@ from typing import Optional, Tuple
 import torch
 from torch import Tensor
 
+from . import _lib, ops
 from .ops import _sparse_attention
 from .utils import (dense_to_ccol_row, dense_to_crow_col, get_sparse_attn_mask, is_kv_cache_efficient,
                     masked_tile_tables, merge_split_fwd_kernel_blocks, multiple_of, split_tile_tables,
@@ -403,17 +404,24 @@ def combine_attn_partitions(*x: Tuple[Tensor, Tensor], hdim=1):
     the head dimension comes right before `dim` -- (batch, seq, heads, dim) with
     hdim=2, or packed (tokens, heads, dim) -- the (.., heads, seq) log-sum-exps
     are transposed to match.  Partitions in which a row saw no key (lse = -inf)
-    get weight 0.
+    get weight 0.  Device tensors go through one fused kernel (and one for the backward);
+    host tensors through the reference's torch expression.
     """
     assert len(x) >= 2 and len(x[0]) == 2
     outputs, weights = list(zip(*x))
+    o0, w0 = outputs[0], weights[0]
+    head_before_dim = (hdim % o0.dim()) == o0.dim() - 2
+    straight = w0.shape == o0.shape[:-1]
+    swapped = w0.dim() >= 2 and w0.transpose(-1, -2).shape == o0.shape[:-1]
+    transposed = swapped and (not straight or (head_before_dim and w0.dim() >= 2))
+    if o0.is_cuda and 2 <= o0.dim() <= 4 and len(x) <= _lib.MAX_PARTITIONS and (straight or swapped):
+        # one fused kernel each way (dk_combine, dk_combine_bwd)
+        return ops.combine_partitions(list(outputs), list(weights), transposed)
+    # host tensors, more than three dims in front of head_dim or more partitions than the
+    # kernel takes: the reference's torch expression
     weights = torch.stack(weights, dim=0)
     outputs = torch.stack(outputs, dim=0)
-    head_before_dim = (hdim % (outputs.dim() - 1)) == outputs.dim() - 3
-    mismatch = weights.shape[1:] != outputs.shape[1:-1]
-    if (head_before_dim and weights.dim() >= 3 and
-            weights.transpose(-1, -2).shape[1:] == outputs.shape[1:-1]) or \
-            (mismatch and weights.transpose(-1, -2).shape[1:] == outputs.shape[1:-1]):
+    if transposed:
         weights = weights.transpose(-1, -2)
     weights = weights.softmax(dim=0)
     weights = torch.where(torch.isnan(weights), torch.zeros_like(weights), weights)

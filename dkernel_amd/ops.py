@@ -601,3 +601,91 @@ class _sparse_attention(torch.autograd.Function):
 
 
 __all__ = ["_sparse_attention", "padded_sparse_attn", "varlen_sparse_attn", "get_qkv_and_pack_mode", "set_impl"]
+
+
+# ---------------------------------------------------------------------------
+# combine_attn_partitions on the device (reference: dkernel/interface.py:303-324)
+# ---------------------------------------------------------------------------
+def _rows3(x: Tensor) -> Tuple[Tuple[int, int, int], Tuple[int, int, int]]:
+    """Extents and element strides of the (at most three) dims in front of head_dim."""
+    lead = x.dim() - 1
+    shape = (1,) * (3 - lead) + tuple(x.shape[:-1])
+    strides = (0,) * (3 - lead) + tuple(x.stride()[:-1])
+    return shape, strides
+
+
+def _fill_combine(args: _lib.CombineArgs, outputs, lses, transposed: bool) -> None:
+    o0 = outputs[0]
+    shape, _ = _rows3(o0)
+    args.num_partitions = len(outputs)
+    args.dtype = _DTYPES[o0.dtype]
+    args.n0, args.n1, args.n2 = shape
+    args.head_dim = o0.size(-1)
+    for i, (o, l) in enumerate(zip(outputs, lses)):
+        args.parts[i] = _lib.Tensor(o.data_ptr(), *_rows3(o)[1])
+        args.lses[i] = _lib.RowVec(l.data_ptr(), *_lse_strides(l, o0.dim() - 1, transposed))
+    args.stream = _stream()
+
+
+def _lse_strides(l: Tensor, lead: int, transposed: bool) -> Tuple[int, int, int]:
+    st = list(l.stride())
+    if transposed:
+        st[-1], st[-2] = st[-2], st[-1]
+    return tuple([0] * (3 - lead) + st)
+
+
+class _CombinePartitions(torch.autograd.Function):
+    """out = sum_p softmax_p(lse_p) * out_p through dk_combine / dk_combine_bwd."""
+
+    @staticmethod
+    def forward(ctx, transposed: bool, n: int, *tensors: Tensor) -> Tensor:
+        outputs = [_unit_last(t) for t in tensors[:n]]
+        lses = [t if t.dtype == torch.float32 else t.float() for t in tensors[n:]]
+        out = torch.empty(outputs[0].shape, dtype=outputs[0].dtype, device=outputs[0].device)
+        args = _lib.CombineArgs()
+        with torch.cuda.device(out.device):
+            _fill_combine(args, outputs, lses, transposed)
+            args.out = _lib.Tensor(out.data_ptr(), *_rows3(out)[1])
+            _lib.check(_lib.lib().dk_combine(C.byref(args)))
+        ctx.save_for_backward(*outputs, *lses)
+        ctx.transposed, ctx.n = transposed, n
+        ctx.lse_dtypes = [t.dtype for t in tensors[n:]]
+        return out
+
+    @staticmethod
+    def backward(ctx, dout: Tensor):
+        n, transposed = ctx.n, ctx.transposed
+        saved = ctx.saved_tensors
+        outputs, lses = saved[:n], saved[n:]
+        dout = _unit_last(dout)
+        dparts = [torch.empty(o.shape, dtype=o.dtype, device=o.device) for o in outputs]
+        dlses = [torch.empty(l.shape, dtype=torch.float32, device=l.device) if ctx.needs_input_grad[2 + n + i] else None
+                 for i, l in enumerate(lses)]
+        args = _lib.CombineArgs()
+        with torch.cuda.device(dout.device):
+            _fill_combine(args, outputs, lses, transposed)
+            args.dout = _lib.Tensor(dout.data_ptr(), *_rows3(dout)[1])
+            for i in range(n):
+                args.dparts[i] = _lib.Tensor(dparts[i].data_ptr(), *_rows3(dparts[i])[1])
+                if dlses[i] is not None:
+                    args.dlses[i] = _lib.RowVec(dlses[i].data_ptr(), *_lse_strides(dlses[i], dout.dim() - 1, transposed))
+            _lib.check(_lib.lib().dk_combine_bwd(C.byref(args)))
+            global last_bwd_kernels
+            last_bwd_kernels = _lib.lib().dk_last_kernels()  # (autograd's thread: the caller's own record is another)
+        dlses = [None if d is None else d.to(dt) for d, dt in zip(dlses, ctx.lse_dtypes)]
+        return (None, None, *dparts, *dlses)
+
+
+def combine_partitions(outputs, lses, transposed: bool) -> Tensor:
+    """Device path of combine_attn_partitions: `outputs` share one shape (.., head_dim) with at
+    most three dims in front of head_dim, `lses` hold one value per row, in the order of the
+    outputs' leading dims or (transposed) with the last two swapped."""
+    o0, l0 = outputs[0], lses[0]
+    assert o0.dtype in _DTYPES, f"unsupported dtype {o0.dtype}"
+    for o, l in zip(outputs, lses):
+        assert o.shape == o0.shape and o.dtype == o0.dtype and o.device == o0.device, "partition outputs differ in shape, dtype or device"
+        assert l.shape == l0.shape and l.device == o0.device, "partition log-sum-exps differ in shape or device"
+    want = tuple(o0.shape[:-1])
+    have = tuple(l0.shape[:-2] + l0.shape[-2:][::-1]) if transposed else tuple(l0.shape)
+    assert have == want, f"log-sum-exps of shape {tuple(l0.shape)} do not line up with outputs of shape {tuple(o0.shape)}"
+    return _CombinePartitions.apply(transposed, len(outputs), *outputs, *lses)

@@ -242,6 +242,38 @@ int dk_bwd(const dk_bwd_args *args);
 /* Scratch that dk_bwd can use for these arguments (0 = none useful; never more than 4 GiB). */
 size_t dk_bwd_workspace_bytes(const dk_bwd_args *args);
 
+/* Merge of attention results computed over disjoint K/V partitions, per row:
+ *     out = sum_p softmax_p(lse_p) * out_p
+ * in fp32, rounded once to the outputs' type.  A partition in which a row saw no key
+ * (lse = -inf) gets weight 0; a row that saw none in any partition gives 0.  Every tensor is
+ * addressed as rows (i0, i1, i2) of head_dim contiguous elements through the three element
+ * strides of its view (named b / h / t in dk_tensor and dk_rowvec), so outputs in (batch,
+ * heads, tokens, dim), (batch, tokens, heads, dim) or packed (tokens, heads, dim) order and
+ * log-sum-exps in (batch, heads, tokens) or (heads, tokens) order all fit; the caller lines
+ * the dims up.  Replaces the torch expression of combine_attn_partitions,
+ * dkernel/interface.py:303-324.
+ *
+ * dk_combine_bwd is its backward: given dout it writes dparts[p] = w_p * dout and (where
+ * dlses[p].ptr is not NULL) dlses[p] = w_p * (<dout, out_p> - <dout, out>).  The reference gets
+ * these from autograd through the same torch expression. */
+#define DK_MAX_PARTITIONS 8
+typedef struct dk_combine_args {
+  int32_t num_partitions; /* 2 .. DK_MAX_PARTITIONS */
+  int32_t dtype;          /* enum dk_dtype of out, dout, parts, dparts */
+  int32_t n0, n1, n2;     /* row extents; i2 runs fastest over the launch */
+  int32_t head_dim;
+  dk_tensor out;                        /* dk_combine: result */
+  dk_tensor dout;                       /* dk_combine_bwd: gradient of the result */
+  dk_tensor parts[DK_MAX_PARTITIONS];   /* out_p */
+  dk_rowvec lses[DK_MAX_PARTITIONS];    /* lse_p, natural log */
+  dk_tensor dparts[DK_MAX_PARTITIONS];  /* dk_combine_bwd: gradients of out_p */
+  dk_rowvec dlses[DK_MAX_PARTITIONS];   /* dk_combine_bwd: gradients of lse_p (ptr may be NULL) */
+  void *stream;                         /* hipStream_t */
+} dk_combine_args;
+
+int dk_combine(const dk_combine_args *args);
+int dk_combine_bwd(const dk_combine_args *args);
+
 #ifdef __cplusplus
 }
 #endif

@@ -35,7 +35,9 @@ static LutView view(const dk_lut &l) {
                  l.max_row_entries, l.sub_block};
 }
 static SeqView view(const dk_seqs &s) {
-  return SeqView{s.batch, s.max_q_len, s.max_k_len, s.packed, s.q_starts, s.q_ends, s.k_starts, s.k_ends};
+  SeqView v{s.batch, s.max_q_len, s.max_k_len, s.packed & 3, s.q_starts, s.q_ends, s.k_starts, s.k_ends};
+  v.zero_outside = (s.packed & 4) && !(s.packed & 1) && s.q_starts ? 1 : 0;  // (without lengths every row holds a query)
+  return v;
 }
 
 static bool vec_aligned(const dk_tensor &t, size_t es) {

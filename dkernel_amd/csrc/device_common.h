@@ -58,6 +58,9 @@ struct SeqView {
   // packed inputs, optional: batch + 1 ints, entry b = work items (q tiles or pairs of q tiles) of
   // the sequences before b, written by a small kernel ahead of the one that reads it
   int32_t *item_offsets = nullptr;
+  // padded inputs: the forward kernels also write the rows of o (zeros) and lse (-inf) that hold
+  // no query of their sequence, so that the caller need not clear the outputs first
+  int32_t zero_outside = 0;
 };
 
 // Paged K/V (decode only): k / v point at page pools, token t of sequence b lives in page
@@ -260,6 +263,48 @@ __device__ __forceinline__ void write_item_offsets(const SeqView &s, int causal,
     }
   }
   if (t == 1023) out[s.batch] = part[1023];
+}
+
+// Padded inputs with SeqView::zero_outside: work item `item` of the `items` that a launch has along
+// the q tiles of one batch entry clears its share of the token rows that hold no query of the
+// sequence (positions outside [q_start, q_start + q_len) of the token dimension), for heads
+// [h0, h0 + nh): o = 0, lse = -inf.  Every item takes part, those without queries too, so the
+// rows are covered whatever the sequence's length.  `vec`: 16-byte stores are legal.
+template <typename T>
+__device__ __forceinline__ void zero_rows_outside(const SeqView &s, const SeqInfo &sq, int item, int items,
+                                                  const TensorView &o, const RowView &lse, int h0, int nh, int D,
+                                                  bool vec, int tid, int nthreads) {
+  const int q_len = sq.q_len > 0 ? sq.q_len : 0;
+  const int outside = s.max_q_len - q_len;
+  if (outside <= 0) return;
+  const int share = (outside + items - 1) / items;
+  const int lo = item * share, hi = min(outside, lo + share);
+  if (lo >= hi) return;
+  auto token = [&](int i) { return i < sq.q_start ? i : i + q_len; };  // i-th row outside the queries
+  // A thread keeps one (head, piece of the row) and walks the rows: the index arithmetic is done
+  // once per thread, not once per store.
+  const bool vec16 = vec && (D * (int)sizeof(T)) % 16 == 0;
+  const int pieces = vec16 ? D * (int)sizeof(T) / 16 : D;  // 16-byte chunks, or elements, per head row
+  const int per_row = nh * pieces;
+  const int groups = nthreads >= per_row ? nthreads / per_row : 1;  // token rows cleared side by side
+  T *ob = (T *)o.ptr + sq.b * o.sb;
+  for (int j = tid; j < per_row * groups; j += nthreads) {
+    const int grp = j / per_row, col = j - grp * per_row;
+    const int hh = col / pieces, c = col - hh * pieces;
+    T *dst = ob + (h0 + hh) * o.sh + (vec16 ? c * (16 / (int)sizeof(T)) : c);
+    for (int i = lo + grp; i < hi; i += groups) {
+      if (vec16)
+        *reinterpret_cast<uint4 *>(dst + (int64_t)token(i) * o.st) = make_uint4(0, 0, 0, 0);
+      else
+        dst[(int64_t)token(i) * o.st] = from_float<T>(0.f);
+    }
+  }
+  if (lse.ptr) {
+    for (int idx = tid; idx < (hi - lo) * nh; idx += nthreads) {
+      const int hh = idx % nh, i = lo + idx / nh;
+      lse.ptr[sq.b * lse.sb + (h0 + hh) * lse.sh + (int64_t)token(i) * lse.st] = -INFINITY;
+    }
+  }
 }
 
 // Maps (tile_x = tile index, bz = batch index) to a sequence and the index of the tile within

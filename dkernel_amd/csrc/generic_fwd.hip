@@ -28,7 +28,10 @@ __global__ __launch_bounds__(256) void generic_fwd_kernel(const FwdParams p) {
   const int tiles_per_block = BM / rows_wg;
   SeqInfo sq;
   int tile;
-  if (!resolve_tile(p.seqs, p.causal, BM, tiles_per_block, blockIdx.x, blockIdx.z, sq, tile)) return;
+  const bool has_rows = resolve_tile(p.seqs, p.causal, BM, tiles_per_block, blockIdx.x, blockIdx.z, sq, tile);
+  if (p.seqs.zero_outside)
+    zero_rows_outside<T>(p.seqs, sq, blockIdx.x, gridDim.x, p.o, p.lse, blockIdx.y, 1, p.D, p.vec_ok, threadIdx.x, 256);
+  if (!has_rows) return;
   const int h = blockIdx.y;
   const int kvh = h / (p.Hq / p.Hkv);
   const int rb = sq.past / BM + tile / tiles_per_block;

@@ -108,7 +108,10 @@ __global__ __launch_bounds__(128) void fwd_kernel(const FwdParams p, int tiles_y
   __shared__ __align__(16) float sV[64 * kLd];
   SeqInfo sq;
   int tile;
-  if (!resolve_tile(p.seqs, p.causal, 64, 1, tiles_y - 1 - (int)blockIdx.y, blockIdx.z, sq, tile)) return;
+  const bool has_rows = resolve_tile(p.seqs, p.causal, 64, 1, tiles_y - 1 - (int)blockIdx.y, blockIdx.z, sq, tile);
+  if (p.seqs.zero_outside)
+    zero_rows_outside<float>(p.seqs, sq, blockIdx.y, tiles_y, p.o, p.lse, blockIdx.x, 1, p.D, p.vec_ok, threadIdx.x, 128);
+  if (!has_rows) return;
   const int rb = sq.past / 64 + tile;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int h = blockIdx.x, kvh = h / (p.Hq / p.Hkv);

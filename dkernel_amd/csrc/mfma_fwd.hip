@@ -76,16 +76,23 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
       u = (first_rb >> 1) + idx;
     } else {
       sq = load_seq(p.seqs, blockIdx.z, p.causal);
-      if (sq.q_len <= 0) return;
       first_rb = sq.past / 64, last_rb = (sq.past + sq.q_len - 1) / 64;
       u = (first_rb >> 1) + tiles_y - 1 - (int)blockIdx.y;
-      if (u > (last_rb >> 1)) return;
+      if (sq.q_len <= 0 || u > (last_rb >> 1)) {  // no rows here: only the share of the padding rows, if asked
+        if (p.seqs.zero_outside)
+          zero_rows_outside<T>(p.seqs, sq, blockIdx.y, tiles_y, p.o, p.lse, blockIdx.x, 1, p.D, p.vec_ok, tid, NT);
+        return;
+      }
     }
     rb = 2 * u + (wave >> 1);
     tile = rb - first_rb;  // outside [0, last_rb - first_rb]: this wave pair has no rows (row_ok false everywhere)
   } else {
     const int ty = tiles_y - 1 - (int)blockIdx.y;  // longest rows first
-    if (!resolve_tile(p.seqs, p.causal, 64, 1, ty, blockIdx.z, sq, tile)) return;
+    if (!resolve_tile(p.seqs, p.causal, 64, 1, ty, blockIdx.z, sq, tile)) {
+      if (p.seqs.zero_outside)  // (never with packed inputs, for which sq is not set here)
+        zero_rows_outside<T>(p.seqs, sq, blockIdx.y, tiles_y, p.o, p.lse, blockIdx.x * G, G, p.D, p.vec_ok, tid, NT);
+      return;
+    }
     rb = sq.past / 64 + tile;
   }
   if constexpr (PAD) {  // the slots of the head dims beyond p.D stay zero for the whole kernel
@@ -389,6 +396,11 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
     store_tile_rows<T, D, PAD>(smem + wave * 32 * TL::kRowBytes, oacc, inv, o_row0, p.o.st, lane, -qi0,
                                sq.q_len - qi0, p.D);
   }
+  // padded inputs: this workgroup's share of the rows that hold no query, behind its own work (at
+  // the start the stores of every workgroup would go out together, ahead of all multiplies)
+  if (p.seqs.zero_outside)
+    zero_rows_outside<T>(p.seqs, sq, blockIdx.y, tiles_y, p.o, p.lse, RP ? blockIdx.x : blockIdx.x * G, RP ? 1 : G, p.D,
+                         p.vec_ok, tid, NT);
   if (!row_ok) return;
   if (p.lse.ptr && g == 0) {
     const float lse = l_run > 0.f ? (m_run + log2f(l_run)) * kLn2 : -INFINITY;

@@ -318,9 +318,12 @@ def padded_sparse_attn(q: Tensor, k: Tensor, v: Tensor, sm_scale: float,
     q, k, v = _unit_last(q), _unit_last(k), _unit_last(v)
     dev = q.device
     _check_out(out, q)
+    # decode writes every row; in padded prefill the kernel clears the padding rows of an output
+    # allocated here itself (bit 2 of dk_seqs.packed), so nothing is filled.  The padding rows of
+    # a caller's `out` stay as they were.
+    clear_padding = out is None and q_len > 1
     if out is None:
-        # decode writes every row; padded prefill leaves the padding rows untouched, so they start at zero
-        out = q.new_empty(q.shape) if q_len == 1 else q.new_zeros(q.shape)
+        out = q.new_empty(q.shape)
 
     if left_paddings is not None:
         assert left_paddings.shape == (batches,)
@@ -339,12 +342,13 @@ def padded_sparse_attn(q: Tensor, k: Tensor, v: Tensor, sm_scale: float,
 
     lse = None
     if return_lse:
-        lse = torch.full((batches, num_heads, q_len), float("-inf"), dtype=torch.float32, device=dev)
+        lse = (torch.empty((batches, num_heads, q_len), dtype=torch.float32, device=dev) if clear_padding or q_len == 1
+               else torch.full((batches, num_heads, q_len), float("-inf"), dtype=torch.float32, device=dev))
     args = _lib.FwdArgs()
     args.q, args.k, args.v, args.o = (_tensor4(x, hdim, seq_dim) for x in (q, k, v, out))
     args.lse = _rowvec(lse)
     args.csr = _lut(sparse_layout, dev, lut_group, lut_max_row)
-    args.seqs = _lib.Seqs(batches, q_len, k_len, 0, q_starts.data_ptr(), q_ends.data_ptr(),
+    args.seqs = _lib.Seqs(batches, q_len, k_len, 4 if clear_padding else 0, q_starts.data_ptr(), q_ends.data_ptr(),
                           k_starts.data_ptr(), k_ends.data_ptr())
     args.num_q_heads, args.num_kv_heads, args.head_dim = num_heads, num_kv_heads, head_size
     args.dtype, args.causal, args.impl = _DTYPES[q.dtype], int(bool(causal)), _impl

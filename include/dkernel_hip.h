@@ -139,7 +139,11 @@ typedef struct dk_seqs {
   int32_t max_k_len;
   int32_t packed;    /* bit 0: sequences share one token dimension (3-D inputs);
                         bit 1 (with bit 0): the caller guarantees exactly one query token per
-                        sequence, which lets dk_fwd take the split-KV decode path */
+                        sequence, which lets dk_fwd take the split-KV decode path;
+                        bit 2 (without bit 0, with the arrays below): dk_fwd also writes the rows
+                        of o (zeros) and lse (-inf) that hold no query of their sequence, so a
+                        padded output need not be cleared first (the reference clears it with
+                        torch.zeros, dkernel/ops/sparse_attn_inference.py:67) */
   const int32_t *q_starts, *q_ends, *k_starts, *k_ends;
 } dk_seqs;
 

@@ -93,7 +93,7 @@ def time_steps(fn, steps, warmup):
 
 
 def quoted_traffic(leg, kernels, version):
-    """(bytes per launch or None, note) for `leg` ("fwd", "bwd", "decode"): the profiled figure if it
+    """(bytes per launch or None, note) for `leg` ("fwd", "bwd", "decode", "combine"): the profiled figure if it
     was taken from the kernels that just ran (names and library version agree), else None."""
     try:
         with open(TRAFFIC_FILE) as f:
@@ -328,9 +328,11 @@ def main():
             _, ec, _ = time_steps(lambda: combine_attn_partitions(*parts), max(10, args.steps), 3)
         # two outputs read, one written (bf16), two log-sum-exps read (fp32)
         comb_bytes = 3 * Tc * Hc * D * 2 + 2 * Tc * Hc * 4
+        comb_kernels = lib.dk_last_kernels().decode()
         extra["combine"] = {"workload": "2 partitions of packed (16384 tokens, 16 heads, d=128) bf16 outputs + fp32 LSE",
-                            "us": round(ec * 1e3, 2), "kernels": lib.dk_last_kernels().decode(),
-                            "roofline": roofline("hbm", comb_bytes, ec, (None, "not profiled"), comb_bytes)}
+                            "us": round(ec * 1e3, 2), "kernels": comb_kernels,
+                            "roofline": roofline("hbm", comb_bytes, ec, quoted_traffic("combine", comb_kernels, version),
+                                                 comb_bytes)}
         out["extra"] = extra
 
     if not args.no_cpu:

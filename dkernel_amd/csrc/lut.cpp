@@ -36,7 +36,7 @@ using dk::fail;
 
 extern "C" {
 
-int dk_version(void) { return 400; /* 0.4.0 */ }
+int dk_version(void) { return 500; /* 0.5.0 */ }
 const char *dk_last_error(void) { return dk::g_err; }
 const char *dk_last_kernels(void) { return dk::g_kernels; }
 

@@ -20,7 +20,7 @@ def _bench():
 def test_record_is_of_this_library_version():
     rec = json.load(open(os.path.join(ROOT, "profiles", "hbm_traffic.json")))
     assert rec["dk_version"] == _lib.lib().dk_version(), "kernels changed version: re-profile and rewrite the record"
-    for leg in ("fwd", "bwd", "decode"):
+    for leg in ("fwd", "bwd", "decode", "combine"):
         assert rec[leg]["kernels"].endswith("; ") and rec[leg]["fetch_bytes"] > 0 and rec[leg]["write_bytes"] >= 0
 
 

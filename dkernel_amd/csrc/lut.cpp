@@ -94,14 +94,27 @@ int dk_csr_count(const int32_t *pattern, int32_t H, int32_t M, int32_t N, int64_
   DK_REQUIRE(pattern && ptr && max_nnz, "NULL argument");
   DK_REQUIRE(H >= 1 && M >= 0 && N >= 0, "bad shape (%d, %d, %d)", H, M, N);
   int32_t mx = 0;
+  // The transpose of a row-major matrix (CSC) is walked in memory order, columns of the output
+  // outermost: along its rows every step would touch another cache line (2.5 s for 8 heads of
+  // 2048 x 2048 blocks against 0.2 s).
+  const bool by_memory = sm < sn;
   for (int h = 0; h < H; ++h) {
     int32_t *p = ptr + (size_t)h * (M + 1);
     p[0] = 0;
-    for (int i = 0; i < M; ++i) {
-      const int32_t *row = pattern + h * sh + i * sm;
-      int32_t c = 0;
-      for (int j = 0; j < N; ++j) c += row[j * sn] != 0;
-      p[i + 1] = p[i] + c;
+    if (by_memory) {
+      for (int i = 0; i < M; ++i) p[i + 1] = 0;
+      for (int j = 0; j < N; ++j) {
+        const int32_t *col = pattern + h * sh + j * sn;
+        for (int i = 0; i < M; ++i) p[i + 1] += col[i * sm] != 0;
+      }
+      for (int i = 0; i < M; ++i) p[i + 1] += p[i];
+    } else {
+      for (int i = 0; i < M; ++i) {
+        const int32_t *row = pattern + h * sh + i * sm;
+        int32_t c = 0;
+        for (int j = 0; j < N; ++j) c += row[j * sn] != 0;
+        p[i + 1] = p[i] + c;
+      }
     }
     if (p[M] > mx) mx = p[M];
   }
@@ -114,19 +127,45 @@ int dk_csr_fill(const int32_t *pattern, int32_t H, int32_t M, int32_t N, int64_t
   dk::clear_error();
   DK_REQUIRE(pattern && (idx || width == 0), "NULL argument");
   DK_REQUIRE(H >= 1 && M >= 0 && N >= 0 && width >= 0, "bad shape");
+  const bool by_memory = sm < sn;  // as in dk_csr_count
+  std::vector<int32_t> cursor;
   for (int h = 0; h < H; ++h) {
     int32_t *o = idx + (size_t)h * width;
     int32_t *ov = val ? val + (size_t)h * width : nullptr;
     int32_t e = 0;
-    for (int i = 0; i < M; ++i) {
-      const int32_t *row = pattern + h * sh + i * sm;
+    if (by_memory) {
+      // first entry of every output row, then one sweep in memory order: column indices reach
+      // each row's list in ascending order
+      cursor.assign((size_t)M + 1, 0);
       for (int j = 0; j < N; ++j) {
-        const int32_t x = row[j * sn];
-        if (x != 0) {
-          if (e >= width) return fail(DK_ERR_INVALID, "width %d too small for head %d", width, h);
-          o[e] = j;
-          if (ov) ov[e] = x;
-          ++e;
+        const int32_t *col = pattern + h * sh + j * sn;
+        for (int i = 0; i < M; ++i) cursor[i + 1] += col[i * sm] != 0;
+      }
+      for (int i = 0; i < M; ++i) cursor[i + 1] += cursor[i];
+      e = cursor[M];
+      if (e > width) return fail(DK_ERR_INVALID, "width %d too small for head %d", width, h);
+      for (int j = 0; j < N; ++j) {
+        const int32_t *col = pattern + h * sh + j * sn;
+        for (int i = 0; i < M; ++i) {
+          const int32_t x = col[i * sm];
+          if (x != 0) {
+            const int32_t at = cursor[i]++;
+            o[at] = j;
+            if (ov) ov[at] = x;
+          }
+        }
+      }
+    } else {
+      for (int i = 0; i < M; ++i) {
+        const int32_t *row = pattern + h * sh + i * sm;
+        for (int j = 0; j < N; ++j) {
+          const int32_t x = row[j * sn];
+          if (x != 0) {
+            if (e >= width) return fail(DK_ERR_INVALID, "width %d too small for head %d", width, h);
+            o[e] = j;
+            if (ov) ov[e] = x;
+            ++e;
+          }
         }
       }
     }

@@ -512,7 +512,8 @@ bool decode_supported(const FwdParams &p, int dtype) {
   return (dtype == DK_BF16 || dtype == DK_F16) && mfma_head_dim_ok(p.D) && lds <= 160 * 1024 && p.csr.block_rows == 64 &&
          p.csr.block_cols == 64 && p.vec_ok &&
          (p.csr.entry_width == 1 || p.csr.sub_block != 0) &&
-         (p.seqs.packed ? (p.seqs.packed & 2) != 0 : p.seqs.max_q_len == 1) && ratio <= 32 && shared_row && p.causal;
+         (p.seqs.packed ? (p.seqs.packed & 2) != 0 : p.seqs.max_q_len == 1) && ratio <= 32 && shared_row && p.causal &&
+         !p.seqs.zero_outside;  // (rows without a query are cleared by the prefill kernels only)
 }
 
 size_t decode_workspace_bytes(const FwdParams &p) {

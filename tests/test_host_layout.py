@@ -348,6 +348,9 @@ def test_c_abi_argument_checks_fail_before_any_launch():
     a = _fake_fwd_args(B=2, Hq=8, Hkv=2, D=128, max_row=10)
     need = lib.dk_fwd_workspace_bytes(ctypes.byref(a))
     assert need > 0 and need % (2 * 8 * 130 * 4) == 0 and need // (2 * 8 * 130 * 4) >= 4
+    a.seqs.packed = 4                          # rows without a query to be cleared: the prefill kernels' job
+    assert lib.dk_fwd_workspace_bytes(ctypes.byref(a)) == 0
+    a.seqs.packed = 0
     a.seqs.max_q_len = 7                       # neither decode nor prefill of the same length
     assert lib.dk_fwd_workspace_bytes(ctypes.byref(a)) == 0
     a = _fake_fwd_args(D=160)                  # head dims above 128 decode on 256-wide tiles

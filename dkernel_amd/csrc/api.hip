@@ -30,9 +30,11 @@ static size_t elem_size(int dtype) { return dtype == DK_F32 ? 4 : 2; }
 static TensorView view(const dk_tensor &t) { return TensorView{t.ptr, t.stride_b, t.stride_h, t.stride_t}; }
 static RowView view(const dk_rowvec &t) { return RowView{t.ptr, t.stride_b, t.stride_h, t.stride_t}; }
 static LutView view(const dk_lut &l) {
-  return LutView{l.ptr, l.idx, l.ptr_stride_h, l.idx_stride_h, l.entry_width, l.num_heads,
-                 l.num_rows, l.block_rows, l.block_cols, l.group < 1 ? 1 : l.group,
-                 l.max_row_entries, l.sub_block};
+  LutView v{l.ptr, l.idx, l.ptr_stride_h, l.idx_stride_h, l.entry_width, l.num_heads,
+            l.num_rows, l.block_rows, l.block_cols, l.group < 1 ? 1 : l.group,
+            l.max_row_entries, l.sub_block};
+  v.order = l.row_order, v.order_sh = l.row_order_stride_h;
+  return v;
 }
 static SeqView view(const dk_seqs &s) {
   SeqView v{s.batch, s.max_q_len, s.max_k_len, s.packed & 3, s.q_starts, s.q_ends, s.k_starts, s.k_ends};

@@ -51,6 +51,8 @@ struct LutView {
   const int32_t *ptr, *idx;
   int64_t ptr_sh, idx_sh;
   int32_t entry_width, num_heads, num_rows, block_rows, block_cols, group, max_row_entries, sub_block;
+  const int32_t *order = nullptr;  // optional: work item i of head h takes table row order[h * order_sh + i]
+  int64_t order_sh = 0;
 };
 struct SeqView {
   int32_t batch, max_q_len, max_k_len, packed;

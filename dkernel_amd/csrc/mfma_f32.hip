@@ -291,10 +291,11 @@ __global__ __launch_bounds__(128) void dkdv_kernel(const BwdParams p) {
   __shared__ __align__(16) float sDo[64 * kLd];
   __shared__ float sLse[64], sDelta[64];
   const SeqInfo sq = load_seq(p.seqs, blockIdx.z, p.causal);
-  const int cb = blockIdx.y;
+  const int kvh = blockIdx.x, ratio = p.Hq / p.Hkv;
+  int cb = blockIdx.y;  // longest columns first when the table gives the order (as in the 16-bit pass)
+  if (p.csc.order) cb = p.csc.order[lut_head(p.csc, kvh * ratio, p.Hq, p.Hkv) * p.csc.order_sh + blockIdx.y];
   if (cb * 64 >= sq.k_len) return;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int kvh = blockIdx.x, ratio = p.Hq / p.Hkv;
   const int n = lane & 31, g = lane >> 5;
   const int key = cb * 64 + wave * 32 + n;
   const bool key_ok = key < sq.k_len;
@@ -403,8 +404,11 @@ int launch_mfma_f32_bwd(const BwdParams &p, hipStream_t stream) {
   DK_NOTE_KERNEL("f32::dq_kernel");
   hipLaunchKernelGGL(f32::dq_kernel, dim3(p.Hq, tiles, s.batch), dim3(128), 0, stream, p, tiles);
   DK_HIP_CHECK(hipGetLastError());
+  BwdParams po = p;  // the order only where heads do not line up with the hardware's 32 workgroup queues
+  if (p.Hkv % 32 == 0) po.csc.order = nullptr;
+  DK_REQUIRE(p.csc.num_rows <= 65535, "sequence too long for one launch");
   DK_NOTE_KERNEL("f32::dkdv_kernel");
-  hipLaunchKernelGGL(f32::dkdv_kernel, dim3(p.Hkv, cblocks, s.batch), dim3(128), 0, stream, p);
+  hipLaunchKernelGGL(f32::dkdv_kernel, dim3(p.Hkv, po.csc.order ? p.csc.num_rows : cblocks, s.batch), dim3(128), 0, stream, po);
   DK_HIP_CHECK(hipGetLastError());
   return DK_OK;
 }

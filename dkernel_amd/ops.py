@@ -87,19 +87,28 @@ def _rowvec(x: Optional[Tensor], strides=None) -> _lib.RowVec:
 _LUT_CACHE = {}
 
 
-def _lut(layout: Tuple[Tensor, Tensor, int, int], device, group: int = 1, max_row: int = 0) -> _lib.Lut:
+def _lut(layout: Tuple[Tensor, Tensor, int, int], device, group: int = 1, max_row: int = 0,
+         longest_first: bool = False) -> _lib.Lut:
     """dk_lut of a layout tuple.  The descriptor of a module's tables never changes, so it is
     built (and checked) once per (tables, hints) and copied from then on (a decode step's host
     time counts).  An entry keeps its two tensors alive, so their addresses cannot be handed to
     other tensors while the entry exists; the caller gets a copy of its own."""
     key = (layout[0].data_ptr(), layout[1].data_ptr(), layout[0].dtype, layout[1].dtype, layout[0].shape,
            layout[1].shape, layout[0].stride(), layout[1].stride(), tuple(int(x) for x in layout[2:]), device, group,
-           max_row)
+           max_row, longest_first)
     hit = _LUT_CACHE.get(key)
     if hit is None:
         if len(_LUT_CACHE) > 256:
             _LUT_CACHE.clear()
-        hit = _LUT_CACHE[key] = (_make_lut(layout, device, group, max_row), layout[0], layout[1])
+        lut = _make_lut(layout, device, group, max_row)
+        order = None
+        if longest_first:
+            # rows of every head by descending length (stable: equal lengths stay in index order),
+            # computed on the device once per table: the dK/dV pass hands its columns out in this order
+            ptr = layout[0] if layout[0].dim() == 2 else layout[0][None]
+            order = torch.argsort(ptr[:, 1:] - ptr[:, :-1], dim=1, descending=True, stable=True).to(torch.int32).contiguous()
+            lut.row_order, lut.row_order_stride_h = order.data_ptr(), order.stride(0)
+        hit = _LUT_CACHE[key] = (lut, layout[0], layout[1], order)
     return _lib.Lut.from_buffer_copy(hit[0])
 
 
@@ -266,7 +275,7 @@ def _backward(ctx, do: Tensor, dlse: Optional[Tensor],
     if masked is not None and _matrix_core_applies(q, k, v, o, do, dq, dk, dv):
         layout_csr, layout_csc = masked[0], masked[1]
     args.csr = _lut(layout_csr, q.device, ctx.lut_group)
-    args.csc = _lut(layout_csc, q.device, ctx.lut_group)
+    args.csc = _lut(layout_csc, q.device, ctx.lut_group, longest_first=True)
     args.seqs = _lib.Seqs(B, Lq, k.size(seq_dim), 0, None, None, None, None)
     args.num_q_heads, args.num_kv_heads, args.head_dim = Hq, k.size(hdim), q.size(-1)
     args.dtype, args.causal, args.impl = _DTYPES[q.dtype], int(bool(ctx.causal)), _impl

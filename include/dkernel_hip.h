@@ -123,6 +123,14 @@ typedef struct dk_lut {
                           f x f pattern blocks, f = 64 / sub_block: bit i * f + j set = rows
                           [i, i+1) * sub_block x columns [j, j+1) * sub_block are attended.  Taken
                           by the matrix-core kernels only. */
+  const int32_t *row_order; /* optional (NULL: ascending): row_order[h * row_order_stride_h + i] is
+                               the table row that the i-th work item of head h takes, a
+                               permutation of 0 .. num_rows-1 with the longest rows first.  Read
+                               by the dK/dV pass for its column table: workgroups are handed to
+                               the shader engines round-robin and in order, so long columns that
+                               recur with a period (vertical strides) otherwise pile up on a few
+                               of them while the rest wait behind a full queue. */
+  int64_t row_order_stride_h;
 } dk_lut;
 
 /* Sequence geometry.  With all four pointers NULL every sequence has

@@ -245,3 +245,26 @@ def test_last_kernels_names_the_path_taken():
         assert ops.last_bwd_kernels.decode().startswith("generic_delta_kernel")
     finally:
         ops.set_impl("auto")
+
+
+@pytest.mark.parametrize("H", [3, 32])
+def test_backward_with_a_table_longer_than_the_keys(H):
+    """The dK/dV pass hands its columns out longest first when the heads do not line up with the
+    hardware's 32 workgroup queues (H = 3; with H = 32 in ascending order): its grid then covers
+    every column of the table, also those beyond the keys of a sequence shorter than max_seqlen."""
+    B, L, D, Lmax = 2, 320, 64, 2048
+    sm = 1 / math.sqrt(D)
+    q, k, v, do = make_qkv(B, L, L, H, H, D, torch.bfloat16, 1, with_do=True)
+    bm = OL.block_mask(H, Lmax, 64, 2, 3)[:, :L // 64, :L // 64]
+    qo, ko, vo = (x.float().requires_grad_() for x in (q, k, v))
+    ro, _ = oracle_fwd(qo, ko, vo, bm, 64, sm)
+    ro.backward(do.float())
+    mod = New(H, Lmax, 64, 2, 3).to(DEV)
+    qd, kd, vd = (x.to(DEV).requires_grad_() for x in (q, k, v))
+    out = mod(qd, kd, vd, sm)
+    out.backward(do.to(DEV))
+    assert b"mfma_dkdv_kernel" in ops.last_bwd_kernels
+    assert_close("O", out, ro, **TOL)
+    assert_close("dQ", qd.grad, qo.grad, **TOL)
+    assert_close("dK", kd.grad, ko.grad, **TOL)
+    assert_close("dV", vd.grad, vo.grad, **TOL)

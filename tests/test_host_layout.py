@@ -33,9 +33,10 @@ def test_library_exports_every_declared_symbol():
 def test_struct_sizes_match_header():
     # natural alignment on x86-64: catches a field added on one side only
     assert ctypes.sizeof(_lib.Tensor) == 32 and ctypes.sizeof(_lib.RowVec) == 32
-    assert ctypes.sizeof(_lib.Lut) == 64 and ctypes.sizeof(_lib.Seqs) == 48
-    assert ctypes.sizeof(_lib.FwdArgs) == 4 * 32 + 32 + 64 + 48 + 7 * 4 + 4 + 3 * 8
-    assert ctypes.sizeof(_lib.BwdArgs) == 8 * 32 + 2 * 32 + 8 + 2 * 64 + 48 + 7 * 4 + 4 + 3 * 8
+    assert ctypes.sizeof(_lib.Lut) == 80 and ctypes.sizeof(_lib.Seqs) == 48
+    assert ctypes.sizeof(_lib.FwdArgs) == 4 * 32 + 32 + 80 + 48 + 7 * 4 + 4 + 3 * 8
+    assert ctypes.sizeof(_lib.BwdArgs) == 8 * 32 + 2 * 32 + 8 + 2 * 80 + 48 + 7 * 4 + 4 + 3 * 8
+    assert ctypes.sizeof(_lib.CombineArgs) == 6 * 4 + 2 * 32 + 4 * 8 * 32 + 8
 
 
 def test_mask_and_luts_match_fixtures(lut_fixtures):
@@ -412,3 +413,24 @@ def test_combine_matches_closed_form():
     for x in l2:
         x[1, 2, 3] = float("-inf")
     assert torch.isfinite(combine_attn_partitions(*zip(o, l2))).all()
+
+
+def test_longest_first_order_of_a_table():
+    """ops._lut(longest_first=True): a permutation of the table rows of every head by descending
+    length, equal lengths in index order (what the dK/dV pass hands out)."""
+    from dkernel_amd import ops
+    from dkernel_amd.utils import dense_to_ccol_row, get_sparse_attn_mask
+    _, mask, _ = get_sparse_attn_mask(4, 1024, block_size=64, local_blocks=2, vert_stride=4, dtype=torch.uint8)
+    ccol, row = dense_to_ccol_row(mask.to(torch.uint8))
+    lut = ops._lut((ccol, row, 64, 64), ccol.device, longest_first=True)
+    assert lut.row_order and lut.row_order_stride_h == 16
+    order = np.ctypeslib.as_array(ctypes.cast(lut.row_order, ctypes.POINTER(ctypes.c_int32)), shape=(ccol.size(0), 16))
+    lens = (ccol[:, 1:] - ccol[:, :-1]).numpy()
+    for h in range(ccol.size(0)):
+        assert sorted(order[h]) == list(range(16))
+        got = lens[h][order[h]]
+        assert (np.diff(got) <= 0).all()
+        for a, b in zip(order[h][:-1], order[h][1:]):
+            assert lens[h][a] > lens[h][b] or a < b
+    plain = ops._lut((ccol, row, 64, 64), ccol.device)
+    assert not plain.row_order

@@ -2,6 +2,7 @@
 
     python benchmark/benchmark_sparse_attn.py [--mode fwd|bwd|both] [--max-log2 16] [--csv out.csv]
         [--batch 4 --heads 16 --head-dim 128 --local-tokens 512 --dtype bfloat16 --impl auto]
+        [--dense-heads 0 [--heads-on-fixed-queues]]
 
 Same sweep as the reference's benchmark/benchmark_sparse_attn.py (its defaults at
 lines 24-40 and 67: batch 4, 16 heads, head_dim 128, local window 512 tokens, block 64,
@@ -9,7 +10,10 @@ bf16, sequence lengths 2^10 .. 2^16, vert_stride in {1, 4, 16}, warm-up 25 / 100
 repetitions), next to PyTorch's dense causal scaled_dot_product_attention when that runs on
 the box.  Prints one table per mode (milliseconds) and optionally writes a CSV.  The shape, the
 dtype and the kernel family (`--impl generic` = the fp32-FMA kernels, `mfma` = matrix cores only)
-can be changed, e.g. for fp32 on the matrix cores against the generic kernels.
+can be changed, e.g. for fp32 on the matrix cores against the generic kernels.  `--dense-heads N`
+makes the last N heads dense (num_dense_heads); `--heads-on-fixed-queues` then switches off the
+rotation of heads over the hardware's workgroup queues that such uneven patterns get, for
+comparison.
 """
 import argparse
 import csv
@@ -24,6 +28,7 @@ from dkernel_amd import LocalStrideSparseAttention, ops  # noqa: E402
 
 B, H, D, BLOCK, LOCAL_TOKENS = 4, 16, 128, 64, 512
 DTYPE = torch.bfloat16
+DENSE_HEADS, FIXED_QUEUES = 0, False
 
 
 def timeit(fn, warmup, reps):
@@ -44,7 +49,9 @@ def bench_one(L, vert, mode, warmup, reps):
     g = torch.Generator(device=dev).manual_seed(20)
     q, k, v, do = (torch.randn(B, L, H, D, generator=g, device=dev, dtype=DTYPE) for _ in range(4))
     sm = 1.0 / math.sqrt(D)
-    mod = LocalStrideSparseAttention(H, L, BLOCK, LOCAL_TOKENS // BLOCK, vert).to(dev)
+    mod = LocalStrideSparseAttention(H, L, BLOCK, LOCAL_TOKENS // BLOCK, vert, num_dense_heads=DENSE_HEADS).to(dev)
+    if FIXED_QUEUES:
+        mod.kwargs["uneven_heads"] = False
     nnz = int(mod.layout_csr_crow[:, -1].sum().item())
     flops = 4.0 * BLOCK * BLOCK * D * nnz * B * (1.0 if mode == "fwd" else 2.5)
     if mode == "fwd":
@@ -73,7 +80,7 @@ def bench_dense(L, mode, warmup, reps):
 
 
 def main():
-    global B, H, D, LOCAL_TOKENS, DTYPE
+    global B, H, D, LOCAL_TOKENS, DTYPE, DENSE_HEADS, FIXED_QUEUES
     defaults = (B, H, D, LOCAL_TOKENS)
     ap = argparse.ArgumentParser()
     ap.add_argument("--mode", default="both", choices=["fwd", "bwd", "both"])
@@ -90,14 +97,18 @@ def main():
     ap.add_argument("--local-tokens", type=int, default=defaults[3])
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float16", "float32"])
     ap.add_argument("--impl", default="auto", choices=["auto", "generic", "mfma"])
+    ap.add_argument("--dense-heads", type=int, default=0)
+    ap.add_argument("--heads-on-fixed-queues", action="store_true")
     args = ap.parse_args()
+    DENSE_HEADS, FIXED_QUEUES = args.dense_heads, args.heads_on_fixed_queues
     B, H, D, LOCAL_TOKENS, DTYPE = args.batch, args.heads, args.head_dim, args.local_tokens, getattr(torch, args.dtype)
     ops.set_impl(args.impl)
     verts = [int(x) for x in args.verts.split(",")]
     rows = []
     for mode in (["fwd", "bwd"] if args.mode == "both" else [args.mode]):
-        print(f"== {mode}: b={B} h={H} d={D} {args.dtype}, block {BLOCK}, local {LOCAL_TOKENS} tokens, kernels: {args.impl}; "
-              "ms (effective TFLOP/s)")
+        print(f"== {mode}: b={B} h={H} d={D} {args.dtype}, block {BLOCK}, local {LOCAL_TOKENS} tokens, kernels: {args.impl}"
+              + (f", last {DENSE_HEADS} heads dense" + (", heads on fixed queues" if FIXED_QUEUES else "") if DENSE_HEADS else "")
+              + "; ms (effective TFLOP/s)")
         print("seqlen".rjust(8) + "".join(f"vert={v}".rjust(22) for v in verts) + "dense sdpa".rjust(14))
         for lg in range(args.min_log2, args.max_log2 + 1):
             L = 1 << lg

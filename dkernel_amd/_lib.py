@@ -32,7 +32,8 @@ class Lut(C.Structure):
     _fields_ = [("ptr", vp), ("idx", vp), ("ptr_stride_h", i64), ("idx_stride_h", i64),
                 ("entry_width", i32), ("num_heads", i32), ("num_rows", i32),
                 ("block_rows", i32), ("block_cols", i32), ("group", i32), ("max_row_entries", i32),
-                ("sub_block", i32), ("row_order", vp), ("row_order_stride_h", i64)]
+                ("sub_block", i32), ("row_order", vp), ("row_order_stride_h", i64),
+                ("uneven_heads", i32), ("reserved", i32)]
 
 
 class Seqs(C.Structure):

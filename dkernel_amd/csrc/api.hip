@@ -34,6 +34,7 @@ static LutView view(const dk_lut &l) {
             l.num_rows, l.block_rows, l.block_cols, l.group < 1 ? 1 : l.group,
             l.max_row_entries, l.sub_block};
   v.order = l.row_order, v.order_sh = l.row_order_stride_h;
+  v.uneven = l.uneven_heads != 0;
   return v;
 }
 static SeqView view(const dk_seqs &s) {

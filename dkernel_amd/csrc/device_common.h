@@ -53,7 +53,33 @@ struct LutView {
   int32_t entry_width, num_heads, num_rows, block_rows, block_cols, group, max_row_entries, sub_block;
   const int32_t *order = nullptr;  // optional: work item i of head h takes table row order[h * order_sh + i]
   int64_t order_sh = 0;
+  int32_t uneven = 0;  // the heads hold clearly different numbers of entries
+  int32_t rot = 0;     // set per launch (head_rotation): 0, or 1 + shift of grid_head()
 };
+
+// Workgroups reach the chip's 32 queues (8 dies x 4 shader engines) by their linear id, in order.
+// With x = head and a head count that is a multiple of 8, 16 or 32 every head stays on the same
+// few queues, and heads of unequal density (dense heads beside sparse ones) leave most of the
+// chip waiting for the busiest queue.  For such tables the head of a workgroup moves on by one
+// with every step in y (every second step once that still takes each head around the queues
+// eight times), so that every queue serves every head in quick succession.  Coarser steps keep
+// more neighbours in y on one die, where they share their K/V (or Q/dO) tiles through its L2,
+// but hand a queue many long workgroups in a row, and the in-order hand-out then stalls behind
+// it: with 32 heads, steps of 4 and 8 measured up to 1.6 x slower, also when every other round
+// ran backwards to even out the growth of the rows along y.  Tables with even heads keep
+// x = head, which shares most (the rotation costs them 8 - 13 %).
+inline int head_rotation(const LutView &l, int gx, int gy) {
+  if (!l.uneven || gx < 2) return 0;
+  return 1 + ((gy >> 3) >= gx ? 1 : 0);
+}
+// Head (or head group) of this workgroup in a grid of (heads, work items, batch).  For every y the
+// map x -> head is a permutation, so each (head, item) pair is still taken exactly once.
+__device__ __forceinline__ int grid_head(const LutView &l) {
+  unsigned x = blockIdx.x;
+  if (l.rot) x = (x + (blockIdx.y >> (l.rot - 1))) % gridDim.x;
+  return __builtin_amdgcn_readfirstlane((int)x);
+}
+
 struct SeqView {
   int32_t batch, max_q_len, max_k_len, packed;
   const int32_t *q_starts, *q_ends, *k_starts, *k_ends;

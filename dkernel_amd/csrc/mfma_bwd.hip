@@ -65,7 +65,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int rh = wave & 1, kh = wave >> 1;  // q-row half, key half
-  const int h = blockIdx.x;
+  const int h = grid_head(p.csr);
   const int kvh = __builtin_amdgcn_readfirstlane(h / (p.Hq / p.Hkv));  // integer division runs on the VALU
   const int m = lane & 31, g = lane >> 5;
   const int row0 = rb * 64 + rh * 32;
@@ -386,7 +386,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, D == 64 
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int ts = wave >> 1, rh = wave & 1;  // which of the two table rows, which half of its 64 q rows
   const int ra = 2 * u, rb = ra + ts;
-  const int h = blockIdx.x;
+  const int h = grid_head(p.csr);
   const int kvh = __builtin_amdgcn_readfirstlane(h / (p.Hq / p.Hkv));  // integer division runs on the VALU
   const int m = lane & 31, g = lane >> 5;
   const int row0 = rb * 64 + rh * 32;
@@ -708,7 +708,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 
   // head_split: one workgroup per q head instead of per kv head; p.dk / p.dv then describe
   // per-q-head partial buffers that a second kernel sums over each kv group
   const int ratio = __builtin_amdgcn_readfirstlane(p.Hq / p.Hkv);  // integer division runs on the VALU
-  const int out_head = blockIdx.x;
+  const int out_head = grid_head(p.csc);
   const int kvh = head_split ? __builtin_amdgcn_readfirstlane(out_head / ratio) : out_head;
   const int gq_first = head_split ? out_head - kvh * ratio : 0;
   const int gq_end = head_split ? gq_first + 1 : ratio;
@@ -1170,12 +1170,16 @@ static int launch_bwd_td(const BwdParams &p, void *workspace, size_t workspace_b
   if constexpr (D <= 128) {  // two table rows per workgroup
     const int pairs = (((past + s.max_q_len - 1) / 64) >> 1) - ((past / 64) >> 1) + 1;
     DK_ALLOW_DYNAMIC_LDS((mfma_dq_pair_kernel<T, D, PAD, SUB>), smem_dq);
-    DK_NOTE_KERNEL("mfma_dq_pair_kernel");
-    hipLaunchKernelGGL((mfma_dq_pair_kernel<T, D, PAD, SUB>), dim3(p.Hq, pairs, s.batch), dim3(256), smem_dq, stream, p, pairs);
+    BwdParams pq = p;
+    pq.csr.rot = head_rotation(p.csr, p.Hq, pairs);  // (uneven heads: dealt to the queues in rotation)
+    DK_NOTE_KERNEL(pq.csr.rot ? "mfma_dq_pair_kernel, heads in rotation" : "mfma_dq_pair_kernel");
+    hipLaunchKernelGGL((mfma_dq_pair_kernel<T, D, PAD, SUB>), dim3(p.Hq, pairs, s.batch), dim3(256), smem_dq, stream, pq, pairs);
   } else {
     DK_ALLOW_DYNAMIC_LDS((mfma_dq_kernel<T, D, PAD, SUB>), smem_dq);
-    DK_NOTE_KERNEL("mfma_dq_kernel");
-    hipLaunchKernelGGL((mfma_dq_kernel<T, D, PAD, SUB>), dim3(p.Hq, tiles, s.batch), dim3(256), smem_dq, stream, p, tiles);
+    BwdParams pq = p;
+    pq.csr.rot = head_rotation(p.csr, p.Hq, tiles);
+    DK_NOTE_KERNEL(pq.csr.rot ? "mfma_dq_kernel, heads in rotation" : "mfma_dq_kernel");
+    hipLaunchKernelGGL((mfma_dq_kernel<T, D, PAD, SUB>), dim3(p.Hq, tiles, s.batch), dim3(256), smem_dq, stream, pq, tiles);
   }
   DK_HIP_CHECK(hipGetLastError());
   // With several q heads per kv head a workgroup per kv head walks all of them, and the longest
@@ -1193,13 +1197,15 @@ static int launch_bwd_td(const BwdParams &p, void *workspace, size_t workspace_b
   if (((per_q_head ? p.Hq : p.Hkv) % 32) == 0) po.csc.order = nullptr;
   // with a hand-out order the grid covers every column of the table (those beyond the keys exit at once)
   const int cblocks = po.csc.order ? p.csc.num_rows : cdiv(s.max_k_len, 64);
+  po.csc.rot = head_rotation(p.csc, per_q_head ? p.Hq : p.Hkv, cblocks);
   if (per_q_head) {
     BwdParams pp = po;
     const int64_t keys = s.max_k_len;
     float *part_k = (float *)workspace, *part_v = part_k + (int64_t)s.batch * p.Hq * keys * p.D;
     pp.dk = TensorView{part_k, p.Hq * keys * p.D, keys * p.D, p.D};
     pp.dv = TensorView{part_v, p.Hq * keys * p.D, keys * p.D, p.D};
-    DK_NOTE_KERNEL("mfma_dkdv_kernel (one workgroup per q head)");
+    DK_NOTE_KERNEL(pp.csc.rot ? "mfma_dkdv_kernel (one workgroup per q head), heads in rotation"
+                              : "mfma_dkdv_kernel (one workgroup per q head)");
     hipLaunchKernelGGL((mfma_dkdv_kernel<T, D, PAD, SUB>), dim3(p.Hq, cblocks, s.batch), dim3(256), smem_dkdv, stream, pp, 1);
     DK_HIP_CHECK(hipGetLastError());
     const int64_t total = (int64_t)s.batch * p.Hkv * keys * (p.D / 8);
@@ -1209,7 +1215,7 @@ static int launch_bwd_td(const BwdParams &p, void *workspace, size_t workspace_b
     DK_HIP_CHECK(hipGetLastError());
     return DK_OK;
   }
-  DK_NOTE_KERNEL("mfma_dkdv_kernel");
+  DK_NOTE_KERNEL(po.csc.rot ? "mfma_dkdv_kernel, heads in rotation" : "mfma_dkdv_kernel");
   hipLaunchKernelGGL((mfma_dkdv_kernel<T, D, PAD, SUB>), dim3(p.Hkv, cblocks, s.batch), dim3(256), smem_dkdv, stream, po, 0);
   DK_HIP_CHECK(hipGetLastError());
   return DK_OK;

@@ -110,11 +110,11 @@ __global__ __launch_bounds__(128) void fwd_kernel(const FwdParams p, int tiles_y
   int tile;
   const bool has_rows = resolve_tile(p.seqs, p.causal, 64, 1, tiles_y - 1 - (int)blockIdx.y, blockIdx.z, sq, tile);
   if (p.seqs.zero_outside)
-    zero_rows_outside<float>(p.seqs, sq, blockIdx.y, tiles_y, p.o, p.lse, blockIdx.x, 1, p.D, p.vec_ok, threadIdx.x, 128);
+    zero_rows_outside<float>(p.seqs, sq, blockIdx.y, tiles_y, p.o, p.lse, grid_head(p.csr), 1, p.D, p.vec_ok, threadIdx.x, 128);
   if (!has_rows) return;
   const int rb = sq.past / 64 + tile;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int h = blockIdx.x, kvh = h / (p.Hq / p.Hkv);
+  const int h = grid_head(p.csr), kvh = h / (p.Hq / p.Hkv);
   const int m = lane & 31, g = lane >> 5;
   const int row0 = rb * 64 + wave * 32;
   const int pos = row0 + m, qi = pos - sq.past;
@@ -225,7 +225,7 @@ __global__ __launch_bounds__(128) void dq_kernel(const BwdParams p, int tiles_y)
   if (tile >= seq_row_blocks(sq, 64)) return;
   const int rb = sq.past / 64 + tile;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int h = blockIdx.x, kvh = h / (p.Hq / p.Hkv);
+  const int h = grid_head(p.csr), kvh = h / (p.Hq / p.Hkv);
   const int m = lane & 31, g = lane >> 5;
   const int row0 = rb * 64 + wave * 32;
   const int pos = row0 + m, qi = pos - sq.past;
@@ -291,7 +291,7 @@ __global__ __launch_bounds__(128) void dkdv_kernel(const BwdParams p) {
   __shared__ __align__(16) float sDo[64 * kLd];
   __shared__ float sLse[64], sDelta[64];
   const SeqInfo sq = load_seq(p.seqs, blockIdx.z, p.causal);
-  const int kvh = blockIdx.x, ratio = p.Hq / p.Hkv;
+  const int kvh = grid_head(p.csc), ratio = p.Hq / p.Hkv;
   int cb = blockIdx.y;  // longest columns first when the table gives the order (as in the 16-bit pass)
   if (p.csc.order) cb = p.csc.order[lut_head(p.csc, kvh * ratio, p.Hq, p.Hkv) * p.csc.order_sh + blockIdx.y];
   if (cb * 64 >= sq.k_len) return;
@@ -386,8 +386,10 @@ int launch_mfma_f32_fwd(const FwdParams &p, hipStream_t stream) {
     tiles = (past + s.max_q_len - 1) / 64 - past / 64 + 1;
   }
   DK_REQUIRE(tiles <= 65535, "too many q tiles for one launch (%d)", tiles);
-  DK_NOTE_KERNEL("f32::fwd_kernel");
-  hipLaunchKernelGGL(f32::fwd_kernel, dim3(p.Hq, tiles, s.packed ? 1 : s.batch), dim3(128), 0, stream, p, tiles);
+  FwdParams pr = p;
+  pr.csr.rot = head_rotation(p.csr, p.Hq, tiles);  // (uneven heads: dealt to the queues in rotation)
+  DK_NOTE_KERNEL(pr.csr.rot ? "f32::fwd_kernel, heads in rotation" : "f32::fwd_kernel");
+  hipLaunchKernelGGL(f32::fwd_kernel, dim3(p.Hq, tiles, s.packed ? 1 : s.batch), dim3(128), 0, stream, pr, tiles);
   DK_HIP_CHECK(hipGetLastError());
   return DK_OK;
 }
@@ -401,14 +403,18 @@ int launch_mfma_f32_bwd(const BwdParams &p, hipStream_t stream) {
   DK_NOTE_KERNEL("f32::delta_kernel");
   hipLaunchKernelGGL(f32::delta_kernel, dim3(cdiv(s.max_q_len, 16), p.Hq, s.batch), dim3(256), 0, stream, p);
   DK_HIP_CHECK(hipGetLastError());
-  DK_NOTE_KERNEL("f32::dq_kernel");
-  hipLaunchKernelGGL(f32::dq_kernel, dim3(p.Hq, tiles, s.batch), dim3(128), 0, stream, p, tiles);
+  BwdParams pq = p;
+  pq.csr.rot = head_rotation(p.csr, p.Hq, tiles);
+  DK_NOTE_KERNEL(pq.csr.rot ? "f32::dq_kernel, heads in rotation" : "f32::dq_kernel");
+  hipLaunchKernelGGL(f32::dq_kernel, dim3(p.Hq, tiles, s.batch), dim3(128), 0, stream, pq, tiles);
   DK_HIP_CHECK(hipGetLastError());
   BwdParams po = p;  // the order only where heads do not line up with the hardware's 32 workgroup queues
   if (p.Hkv % 32 == 0) po.csc.order = nullptr;
   DK_REQUIRE(p.csc.num_rows <= 65535, "sequence too long for one launch");
-  DK_NOTE_KERNEL("f32::dkdv_kernel");
-  hipLaunchKernelGGL(f32::dkdv_kernel, dim3(p.Hkv, po.csc.order ? p.csc.num_rows : cblocks, s.batch), dim3(128), 0, stream, po);
+  const int columns = po.csc.order ? p.csc.num_rows : cblocks;
+  po.csc.rot = head_rotation(p.csc, p.Hkv, columns);
+  DK_NOTE_KERNEL(po.csc.rot ? "f32::dkdv_kernel, heads in rotation" : "f32::dkdv_kernel");
+  hipLaunchKernelGGL(f32::dkdv_kernel, dim3(p.Hkv, columns, s.batch), dim3(128), 0, stream, po);
   DK_HIP_CHECK(hipGetLastError());
   return DK_OK;
 }

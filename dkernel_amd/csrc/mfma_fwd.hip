@@ -80,7 +80,7 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
       u = (first_rb >> 1) + tiles_y - 1 - (int)blockIdx.y;
       if (sq.q_len <= 0 || u > (last_rb >> 1)) {  // no rows here: only the share of the padding rows, if asked
         if (p.seqs.zero_outside)
-          zero_rows_outside<T>(p.seqs, sq, blockIdx.y, tiles_y, p.o, p.lse, blockIdx.x, 1, p.D, p.vec_ok, tid, NT);
+          zero_rows_outside<T>(p.seqs, sq, blockIdx.y, tiles_y, p.o, p.lse, grid_head(p.csr), 1, p.D, p.vec_ok, tid, NT);
         return;
       }
     }
@@ -90,7 +90,7 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
     const int ty = tiles_y - 1 - (int)blockIdx.y;  // longest rows first
     if (!resolve_tile(p.seqs, p.causal, 64, 1, ty, blockIdx.z, sq, tile)) {
       if (p.seqs.zero_outside)  // (never with packed inputs, for which sq is not set here)
-        zero_rows_outside<T>(p.seqs, sq, blockIdx.y, tiles_y, p.o, p.lse, blockIdx.x * G, G, p.D, p.vec_ok, tid, NT);
+        zero_rows_outside<T>(p.seqs, sq, blockIdx.y, tiles_y, p.o, p.lse, grid_head(p.csr) * G, G, p.D, p.vec_ok, tid, NT);
       return;
     }
     rb = sq.past / 64 + tile;
@@ -99,7 +99,8 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
     zero_tiles<NT>(smem, 2 * S::kStage, tid);
     __syncthreads();
   }
-  const int h = RP ? blockIdx.x : blockIdx.x * G + (wave >> 1);
+  const int hx = grid_head(p.csr);  // head (row pairs) or group of G heads of this workgroup
+  const int h = RP ? hx : hx * G + (wave >> 1);
   const int kvh = __builtin_amdgcn_readfirstlane(h / (p.Hq / p.Hkv));  // integer division runs on the VALU
   const int m = lane & 31, g = lane >> 5;
   const int row0 = rb * 64 + (wave & 1) * 32;  // first absolute position of this wave
@@ -119,7 +120,7 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
     }
   }
 
-  const int lh = lut_head(p.csr, RP ? blockIdx.x : blockIdx.x * G, p.Hq, p.Hkv);
+  const int lh = lut_head(p.csr, RP ? hx : hx * G, p.Hq, p.Hkv);
   int e0 = 0, e1 = 0;
   int emid = 0;  // RP: entries [e0, emid) are row 2u, [emid, e1) row 2u + 1 (consecutive rows follow each other)
   if constexpr (RP) {
@@ -399,7 +400,7 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
   // padded inputs: this workgroup's share of the rows that hold no query, behind its own work (at
   // the start the stores of every workgroup would go out together, ahead of all multiplies)
   if (p.seqs.zero_outside)
-    zero_rows_outside<T>(p.seqs, sq, blockIdx.y, tiles_y, p.o, p.lse, RP ? blockIdx.x : blockIdx.x * G, RP ? 1 : G, p.D,
+    zero_rows_outside<T>(p.seqs, sq, blockIdx.y, tiles_y, p.o, p.lse, RP ? hx : hx * G, RP ? 1 : G, p.D,
                          p.vec_ok, tid, NT);
   if (!row_ok) return;
   if (p.lse.ptr && g == 0) {
@@ -490,6 +491,13 @@ bool mfma_fwd_supported(const FwdParams &p, int dtype) {
          p.scale_log2 > 0.f;  // the row maximum is taken before scaling (a scale <= 0 runs on the generic kernels)
 }
 
+// The parameters of a launch of (gx heads or head groups) x (gy work items): tables with uneven
+// heads get their head rotation.
+static FwdParams for_grid(FwdParams p, int gx, int gy) {
+  p.csr.rot = head_rotation(p.csr, gx, gy);
+  return p;
+}
+
 // Several q heads per workgroup (G = 2 or 4 heads that share a kv head and a table row).
 template <typename T, int D, int G, bool PAD>
 static int launch_tdg(const FwdParams &p, dim3 grid, int tiles_y, hipStream_t stream) {
@@ -497,8 +505,10 @@ static int launch_tdg(const FwdParams &p, dim3 grid, int tiles_y, hipStream_t st
   DK_ALLOW_DYNAMIC_LDS((mfma_fwd_kernel<T, D, G, PAD, false>), smem);
   grid.x = p.Hq / G;
   if (int rc = launch_item_offsets(p, false, stream)) return rc;
-  DK_NOTE_KERNEL("mfma_fwd_kernel");
-  hipLaunchKernelGGL((mfma_fwd_kernel<T, D, G, PAD, false>), grid, dim3(128 * G), smem, stream, p, tiles_y);
+  const FwdParams pr = for_grid(p, grid.x, grid.y);
+  DK_NOTE_KERNEL(pr.csr.rot ? "mfma_fwd_kernel, heads in rotation" : "mfma_fwd_kernel");
+  hipLaunchKernelGGL((mfma_fwd_kernel<T, D, G, PAD, false>), grid, dim3(128 * G), smem, stream,
+                     pr, tiles_y);
   DK_HIP_CHECK(hipGetLastError());
   return DK_OK;
 }
@@ -523,9 +533,10 @@ static int launch_row_pairs(const FwdParams &p, hipStream_t stream) {
   }
   DK_REQUIRE(pairs <= 65535, "too many q tiles for one launch (%d)", pairs);
   if (int rc = launch_item_offsets(p, true, stream)) return rc;
-  DK_NOTE_KERNEL("mfma_fwd_kernel");
+  const FwdParams pr = for_grid(p, p.Hq, pairs);
+  DK_NOTE_KERNEL(pr.csr.rot ? "mfma_fwd_kernel, heads in rotation" : "mfma_fwd_kernel");
   hipLaunchKernelGGL((mfma_fwd_kernel<T, D, 2, PAD, true>), dim3(p.Hq, pairs, s.packed ? 1 : s.batch), dim3(256), smem,
-                     stream, p, pairs);
+                     stream, pr, pairs);
   DK_HIP_CHECK(hipGetLastError());
   return DK_OK;
 }
@@ -546,8 +557,10 @@ static int launch_sub_g(const FwdParams &p, dim3 grid, int tiles_y, hipStream_t 
   DK_ALLOW_DYNAMIC_LDS((mfma_fwd_kernel<T, D, G, PAD, false, true>), smem);
   grid.x = p.Hq / G;
   if (int rc = launch_item_offsets(p, false, stream)) return rc;
-  DK_NOTE_KERNEL("mfma_fwd_kernel");
-  hipLaunchKernelGGL((mfma_fwd_kernel<T, D, G, PAD, false, true>), grid, dim3(128 * G), smem, stream, p, tiles_y);
+  const FwdParams pr = for_grid(p, grid.x, grid.y);
+  DK_NOTE_KERNEL(pr.csr.rot ? "mfma_fwd_kernel, heads in rotation" : "mfma_fwd_kernel");
+  hipLaunchKernelGGL((mfma_fwd_kernel<T, D, G, PAD, false, true>), grid, dim3(128 * G), smem, stream,
+                     pr, tiles_y);
   DK_HIP_CHECK(hipGetLastError());
   return DK_OK;
 }
@@ -570,8 +583,10 @@ static int launch_256_g(const FwdParams &p, dim3 grid, int tiles_y, hipStream_t 
   DK_ALLOW_DYNAMIC_LDS((mfma_fwd_kernel<T, 256, G, true, false, SUB>), smem);
   grid.x = p.Hq / G;
   if (int rc = launch_item_offsets(p, false, stream)) return rc;
-  DK_NOTE_KERNEL("mfma_fwd_kernel");
-  hipLaunchKernelGGL((mfma_fwd_kernel<T, 256, G, true, false, SUB>), grid, dim3(128 * G), smem, stream, p, tiles_y);
+  const FwdParams pr = for_grid(p, grid.x, grid.y);
+  DK_NOTE_KERNEL(pr.csr.rot ? "mfma_fwd_kernel, heads in rotation" : "mfma_fwd_kernel");
+  hipLaunchKernelGGL((mfma_fwd_kernel<T, 256, G, true, false, SUB>), grid, dim3(128 * G), smem, stream,
+                     pr, tiles_y);
   DK_HIP_CHECK(hipGetLastError());
   return DK_OK;
 }

@@ -44,6 +44,16 @@ def _identical_head_run(pattern: Tensor) -> int:
     return 1
 
 
+def _uneven_heads(pattern: Tensor) -> bool:
+    """True when some head of the pattern holds clearly more blocks than the average head (a
+    fifth more: below that, keeping each head on its own workgroup queues shares more tiles
+    through the caches than spreading the heads would gain)."""
+    if pattern.size(0) < 2 or pattern.stride(0) == 0:
+        return False
+    counts = pattern.reshape(pattern.size(0), -1).sum(1, dtype=torch.int64).cpu()
+    return bool(counts.max() * counts.numel() > 1.2 * counts.sum())
+
+
 class SparseAttention(torch.nn.Module):
     """Block-sparse attention over a user-given block pattern.
 
@@ -120,6 +130,10 @@ class SparseAttention(torch.nn.Module):
         # q heads whose patterns are identical (a GQA group) can share K/V tiles on chip
         self.lut_group = _identical_head_run(sparse_pattern)
         self.kwargs['lut_group'] = self.lut_group
+        # heads that hold clearly different numbers of blocks (dense heads beside sparse ones): the
+        # prefill and backward kernels then deal the heads to the hardware's workgroup queues in
+        # rotation, so that no part of the chip is left with the dense heads alone
+        self.kwargs['uneven_heads'] = _uneven_heads(sparse_pattern)
 
         if not causal:
             # merged q tiles are a causal-only optimisation

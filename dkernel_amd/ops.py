@@ -88,19 +88,20 @@ _LUT_CACHE = {}
 
 
 def _lut(layout: Tuple[Tensor, Tensor, int, int], device, group: int = 1, max_row: int = 0,
-         longest_first: bool = False) -> _lib.Lut:
+         longest_first: bool = False, uneven: bool = False) -> _lib.Lut:
     """dk_lut of a layout tuple.  The descriptor of a module's tables never changes, so it is
     built (and checked) once per (tables, hints) and copied from then on (a decode step's host
     time counts).  An entry keeps its two tensors alive, so their addresses cannot be handed to
     other tensors while the entry exists; the caller gets a copy of its own."""
     key = (layout[0].data_ptr(), layout[1].data_ptr(), layout[0].dtype, layout[1].dtype, layout[0].shape,
            layout[1].shape, layout[0].stride(), layout[1].stride(), tuple(int(x) for x in layout[2:]), device, group,
-           max_row, longest_first)
+           max_row, longest_first, uneven)
     hit = _LUT_CACHE.get(key)
     if hit is None:
         if len(_LUT_CACHE) > 256:
             _LUT_CACHE.clear()
         lut = _make_lut(layout, device, group, max_row)
+        lut.uneven_heads = int(bool(uneven))
         order = None
         if longest_first:
             # rows of every head by descending length (stable: equal lengths stay in index order),
@@ -196,7 +197,8 @@ def _forward(ctx, q: Tensor, k: Tensor, v: Tensor, sm_scale: float,
              causal=True,
              split_qkv=None,
              lut_group: int = 1,
-             lut_max_row: int = 0) -> Tuple[Tensor, Optional[Tensor]]:
+             lut_max_row: int = 0,
+             uneven_heads: bool = False) -> Tuple[Tensor, Optional[Tensor]]:
     """Unpadded 4-D forward (training, prefill, single-token decode).
     Reference: dkernel/ops/sparse_attn_fwd.py:383-567.  `d_splits` is accepted
     and ignored (a Triton shared-memory workaround)."""
@@ -223,7 +225,7 @@ def _forward(ctx, q: Tensor, k: Tensor, v: Tensor, sm_scale: float,
     args = _lib.FwdArgs()
     args.q, args.k, args.v, args.o = (_tensor4(x, hdim, seq_dim) for x in (q, k, v, o))
     args.lse = _rowvec(lse)
-    args.csr = _lut(layout_csr, q.device, lut_group, lut_max_row)
+    args.csr = _lut(layout_csr, q.device, lut_group, lut_max_row, uneven=uneven_heads)
     args.seqs = _lib.Seqs(q.size(0), qlen, klen, 0, None, None, None, None)
     args.num_q_heads, args.num_kv_heads, args.head_dim = num_heads, num_kv_heads, q.size(-1)
     args.dtype, args.causal, args.impl = _DTYPES[q.dtype], int(bool(causal)), _impl
@@ -237,6 +239,7 @@ def _forward(ctx, q: Tensor, k: Tensor, v: Tensor, sm_scale: float,
     ctx.hdim = hdim
     ctx.causal = causal
     ctx.lut_group = lut_group
+    ctx.uneven_heads = uneven_heads
     return o, (lse if return_lse else None)
 
 
@@ -274,8 +277,9 @@ def _backward(ctx, do: Tensor, dlse: Optional[Tensor],
     masked = getattr(ctx, "masked_layouts", None)
     if masked is not None and _matrix_core_applies(q, k, v, o, do, dq, dk, dv):
         layout_csr, layout_csc = masked[0], masked[1]
-    args.csr = _lut(layout_csr, q.device, ctx.lut_group)
-    args.csc = _lut(layout_csc, q.device, ctx.lut_group, longest_first=True)
+    uneven = getattr(ctx, "uneven_heads", False)
+    args.csr = _lut(layout_csr, q.device, ctx.lut_group, uneven=uneven)
+    args.csc = _lut(layout_csc, q.device, ctx.lut_group, longest_first=True, uneven=uneven)
     args.seqs = _lib.Seqs(B, Lq, k.size(seq_dim), 0, None, None, None, None)
     args.num_q_heads, args.num_kv_heads, args.head_dim = Hq, k.size(hdim), q.size(-1)
     args.dtype, args.causal, args.impl = _DTYPES[q.dtype], int(bool(ctx.causal)), _impl
@@ -304,7 +308,8 @@ def padded_sparse_attn(q: Tensor, k: Tensor, v: Tensor, sm_scale: float,
                        causal: bool = True,
                        return_lse: bool = False,
                        lut_group: int = 1,
-                       lut_max_row: int = 0):
+                       lut_max_row: int = 0,
+                       uneven_heads: bool = False):
     """4-D inputs with left paddings and / or explicit sequence lengths; q has
     either one token per sequence (decode) or the same padded length as k.
     Reference: dkernel/ops/sparse_attn_inference.py:10-147.  Padding rows of
@@ -356,7 +361,7 @@ def padded_sparse_attn(q: Tensor, k: Tensor, v: Tensor, sm_scale: float,
     args = _lib.FwdArgs()
     args.q, args.k, args.v, args.o = (_tensor4(x, hdim, seq_dim) for x in (q, k, v, out))
     args.lse = _rowvec(lse)
-    args.csr = _lut(sparse_layout, dev, lut_group, lut_max_row)
+    args.csr = _lut(sparse_layout, dev, lut_group, lut_max_row, uneven=uneven_heads and q_len > 1)
     args.seqs = _lib.Seqs(batches, q_len, k_len, 4 if clear_padding else 0, q_starts.data_ptr(), q_ends.data_ptr(),
                           k_starts.data_ptr(), k_ends.data_ptr())
     args.num_q_heads, args.num_kv_heads, args.head_dim = num_heads, num_kv_heads, head_size
@@ -446,7 +451,8 @@ def varlen_sparse_attn(q: Tensor, k: Tensor, v: Tensor,
                        causal: bool = True,
                        return_lse: bool = False,
                        lut_group: int = 1,
-                       lut_max_row: int = 0):
+                       lut_max_row: int = 0,
+                       uneven_heads: bool = False):
     """Packed variable-length inputs (total_tokens, heads, head_dim) with
     cumulative sequence lengths.  Reference:
     dkernel/ops/sparse_attn_inference.py:150-287.  The query tokens of a
@@ -483,7 +489,7 @@ def varlen_sparse_attn(q: Tensor, k: Tensor, v: Tensor,
     args = _lib.FwdArgs()
     args.q, args.k, args.v, args.o = (_tensor3(x) for x in (q, k, v, out))
     args.lse = _rowvec(lse, (0, lse.stride(0), lse.stride(1))) if lse is not None else _rowvec(None)
-    args.csr = _lut(sparse_layout, dev, lut_group, lut_max_row)
+    args.csr = _lut(sparse_layout, dev, lut_group, lut_max_row, uneven=uneven_heads and not single_query)
     isz = cu_q.element_size()
     args.seqs = _lib.Seqs(batch_size, q.size(0), k.size(0), 3 if single_query else 1,
                           cu_q.data_ptr(), cu_q.data_ptr() + isz, cu_k.data_ptr(), cu_k.data_ptr() + isz)
@@ -565,7 +571,8 @@ class _sparse_attention(torch.autograd.Function):
             ctx.message = "Currently does not suppoort variable length inputs. WIP."
             res = varlen_sparse_attn(q, k, v, inf_kwargs["cu_seqlen_k"], inf_kwargs.get("cu_seqlen_q", None),
                                      sm_scale, layout_csr, max_seqlen=max_seqlen, causal=causal,
-                                     out=kwargs.get("out", None), return_lse=return_lse, lut_group=lut_group, lut_max_row=lut_max_row)
+                                     out=kwargs.get("out", None), return_lse=return_lse, lut_group=lut_group, lut_max_row=lut_max_row,
+                                     uneven_heads=kwargs.get("uneven_heads", False))
             output, lse = res if return_lse else (res, None)
         else:
             assert k.size(seq_dim) <= max_seqlen, \
@@ -580,14 +587,14 @@ class _sparse_attention(torch.autograd.Function):
                                          seqlens=seqlens, seq_dim=seq_dim, max_seqlen=max_seqlen,
                                          out=kwargs.get("out", None),
                                          causal=causal, return_lse=return_lse, lut_group=lut_group,
-                                         lut_max_row=lut_max_row)
+                                         lut_max_row=lut_max_row, uneven_heads=kwargs.get("uneven_heads", False))
                 output, lse = res if return_lse else (res, None)
             else:
                 ctx.support_backward = True
                 ctx.message = ""
                 fwd_kwargs = {k_: v_ for k_, v_ in kwargs.items()
                               if k_ in ("inference", "out", "d_splits", "max_seqlen", "return_lse",
-                                        "causal", "split_qkv", "lut_group")}
+                                        "causal", "split_qkv", "lut_group", "uneven_heads")}
                 fwd_kwargs["lut_max_row"] = lut_max_row
                 output, lse = _forward(ctx, q, k, v, sm_scale, layout_csr, seq_dim=seq_dim, **fwd_kwargs)
         return output, lse

@@ -131,6 +131,13 @@ typedef struct dk_lut {
                                recur with a period (vertical strides) otherwise pile up on a few
                                of them while the rest wait behind a full queue. */
   int64_t row_order_stride_h;
+  int32_t uneven_heads; /* nonzero: the heads of the table hold clearly different numbers of entries
+                           (dense heads beside sparse ones).  The matrix-core prefill and backward
+                           kernels then deal the heads to the workgroup queues in rotation instead
+                           of one head per queue, so that no part of the chip is left with the
+                           dense heads alone; with even heads (0) a fixed head per queue shares more
+                           tiles through the caches.  Results do not depend on it. */
+  int32_t reserved;     /* 0 */
 } dk_lut;
 
 /* Sequence geometry.  With all four pointers NULL every sequence has

@@ -14,7 +14,8 @@ import torch
 
 import dkernel_amd
 from dkernel_amd import _lib, utils as U
-from dkernel_amd.interface import LocalStrideSparseAttention, SparseAttention, combine_attn_partitions
+from dkernel_amd.interface import (LocalStrideSparseAttention, SparseAttention, _uneven_heads,
+                                   combine_attn_partitions)
 from oracle import layout as OL
 from conftest import ROOT, mask_kwargs
 
@@ -33,9 +34,9 @@ def test_library_exports_every_declared_symbol():
 def test_struct_sizes_match_header():
     # natural alignment on x86-64: catches a field added on one side only
     assert ctypes.sizeof(_lib.Tensor) == 32 and ctypes.sizeof(_lib.RowVec) == 32
-    assert ctypes.sizeof(_lib.Lut) == 80 and ctypes.sizeof(_lib.Seqs) == 48
-    assert ctypes.sizeof(_lib.FwdArgs) == 4 * 32 + 32 + 80 + 48 + 7 * 4 + 4 + 3 * 8
-    assert ctypes.sizeof(_lib.BwdArgs) == 8 * 32 + 2 * 32 + 8 + 2 * 80 + 48 + 7 * 4 + 4 + 3 * 8
+    assert ctypes.sizeof(_lib.Lut) == 88 and ctypes.sizeof(_lib.Seqs) == 48
+    assert ctypes.sizeof(_lib.FwdArgs) == 4 * 32 + 32 + 88 + 48 + 7 * 4 + 4 + 3 * 8
+    assert ctypes.sizeof(_lib.BwdArgs) == 8 * 32 + 2 * 32 + 8 + 2 * 88 + 48 + 7 * 4 + 4 + 3 * 8
     assert ctypes.sizeof(_lib.CombineArgs) == 6 * 4 + 2 * 32 + 4 * 8 * 32 + 8
 
 
@@ -434,3 +435,13 @@ def test_longest_first_order_of_a_table():
             assert lens[h][a] > lens[h][b] or a < b
     plain = ops._lut((ccol, row, 64, 64), ccol.device)
     assert not plain.row_order
+
+
+def test_which_patterns_count_as_uneven():
+    mask = lambda **kw: torch.from_numpy(OL.block_mask(8, 2048, 64, 2, 4, **kw).astype("uint8"))  # noqa: E731
+    assert not _uneven_heads(mask())
+    assert not _uneven_heads(mask(homo_head=True))
+    assert not _uneven_heads(mask(head_sliding_offset=1))
+    assert _uneven_heads(mask(num_dense_heads=1))
+    assert _uneven_heads(mask(num_dense_heads=4))
+    assert not _uneven_heads(mask(num_dense_heads=8))  # every head dense: even again

@@ -107,3 +107,28 @@ def test_padded_and_packed_prefill_do_not_depend_on_the_rotation(Hq, Hkv, D):
         results.append(got)
     for a, b in zip(*results):
         assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("H,L", [(32, 16384), (16, 8192)])
+def test_long_contexts_do_not_depend_on_the_rotation(H, L):
+    """At the lengths where the rotation pays (and where the dK/dV grid is long enough for steps of
+    two): forward and backward are bit-identical with and without it."""
+    print(f"case H={H} L={L}", flush=True)
+    D = 128
+    sm = 1 / math.sqrt(D)
+    mod = New(H, L, 64, 8, 8, num_dense_heads=H // 8).to(DEV)
+    assert mod.kwargs["uneven_heads"]
+    g = torch.Generator(device=DEV).manual_seed(20)
+    q, k, v, do = (torch.randn(1, L, H, D, generator=g, device=DEV).to(torch.bfloat16) for _ in range(4))
+    results = []
+    for uneven in (True, False):
+        mod.kwargs["uneven_heads"] = uneven
+        qd, kd, vd = (x.clone().requires_grad_() for x in (q, k, v))
+        out, lse = mod(qd, kd, vd, sm, return_lse=True)
+        assert (b"heads in rotation" in _last_fwd()) == uneven
+        out.backward(do)
+        assert ops.last_bwd_kernels.count(b"heads in rotation") == (2 if uneven else 0)
+        results.append((out, lse, qd.grad, kd.grad, vd.grad))
+    assert torch.isfinite(results[0][0].float()).all() and torch.isfinite(results[0][2].float()).all()
+    for a, b in zip(*results):
+        assert torch.equal(a, b)

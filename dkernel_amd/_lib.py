@@ -33,7 +33,7 @@ class Lut(C.Structure):
                 ("entry_width", i32), ("num_heads", i32), ("num_rows", i32),
                 ("block_rows", i32), ("block_cols", i32), ("group", i32), ("max_row_entries", i32),
                 ("sub_block", i32), ("row_order", vp), ("row_order_stride_h", i64),
-                ("uneven_heads", i32), ("reserved", i32)]
+                ("uneven_heads", i32), ("reserved", i32), ("pair_order", vp)]
 
 
 class Seqs(C.Structure):

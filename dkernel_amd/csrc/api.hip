@@ -33,7 +33,7 @@ static LutView view(const dk_lut &l) {
   LutView v{l.ptr, l.idx, l.ptr_stride_h, l.idx_stride_h, l.entry_width, l.num_heads,
             l.num_rows, l.block_rows, l.block_cols, l.group < 1 ? 1 : l.group,
             l.max_row_entries, l.sub_block};
-  v.order = l.row_order, v.order_sh = l.row_order_stride_h;
+  v.order = l.row_order, v.pair_order = l.pair_order, v.order_sh = l.row_order_stride_h;
   v.uneven = l.uneven_heads != 0;
   return v;
 }

@@ -52,6 +52,7 @@ struct LutView {
   int64_t ptr_sh, idx_sh;
   int32_t entry_width, num_heads, num_rows, block_rows, block_cols, group, max_row_entries, sub_block;
   const int32_t *order = nullptr;  // optional: work item i of head h takes table row order[h * order_sh + i]
+  const int32_t *pair_order = nullptr;  // optional: ... or the rows 2u, 2u + 1 with u = pair_order[h * order_sh + i]
   int64_t order_sh = 0;
   int32_t uneven = 0;  // the heads hold clearly different numbers of entries
   int32_t rot = 0;     // set per launch (head_rotation): 0, or 1 + shift of grid_head()

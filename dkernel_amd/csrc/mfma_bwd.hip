@@ -59,13 +59,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 
   extern __shared__ __align__(16) char smem[];
 
   const SeqInfo sq = load_seq(p.seqs, blockIdx.z, p.causal);
-  const int tile = tiles_y - 1 - (int)blockIdx.y;
-  if (tile >= seq_row_blocks(sq, 64)) return;
+  const int h = grid_head(p.csr);
+  int tile = tiles_y - 1 - (int)blockIdx.y;  // longest rows first (of a causal pattern)
+  if (p.csr.order)  // the table's own order, longest rows first (the grid then covers every row of it)
+    tile = scalar_load(p.csr.order + lut_head(p.csr, h, p.Hq, p.Hkv) * p.csr.order_sh + blockIdx.y) - sq.past / 64;
+  if (tile < 0 || tile >= seq_row_blocks(sq, 64)) return;
   const int rb = sq.past / 64 + tile;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int rh = wave & 1, kh = wave >> 1;  // q-row half, key half
-  const int h = grid_head(p.csr);
   const int kvh = __builtin_amdgcn_readfirstlane(h / (p.Hq / p.Hkv));  // integer division runs on the VALU
   const int m = lane & 31, g = lane >> 5;
   const int row0 = rb * 64 + rh * 32;
@@ -380,13 +382,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, D == 64 
   const SeqInfo sq = load_seq(p.seqs, blockIdx.z, p.causal);
   if (sq.q_len <= 0) return;
   const int first_rb = sq.past / 64, last_rb = (sq.past + sq.q_len - 1) / 64;
-  const int u = (first_rb >> 1) + pairs_y - 1 - (int)blockIdx.y;  // longest rows first
-  if (u > (last_rb >> 1)) return;
+  const int h = grid_head(p.csr);
+  int u = (first_rb >> 1) + pairs_y - 1 - (int)blockIdx.y;  // longest rows first (of a causal pattern)
+  if (p.csr.pair_order)  // the table's own order, longest pairs first (the grid then covers every pair of it)
+    u = scalar_load(p.csr.pair_order + lut_head(p.csr, h, p.Hq, p.Hkv) * p.csr.order_sh + blockIdx.y);
+  if (u > (last_rb >> 1) || u < (first_rb >> 1)) return;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int ts = wave >> 1, rh = wave & 1;  // which of the two table rows, which half of its 64 q rows
   const int ra = 2 * u, rb = ra + ts;
-  const int h = grid_head(p.csr);
   const int kvh = __builtin_amdgcn_readfirstlane(h / (p.Hq / p.Hkv));  // integer division runs on the VALU
   const int m = lane & 31, g = lane >> 5;
   const int row0 = rb * 64 + rh * 32;
@@ -1165,21 +1169,25 @@ static int launch_bwd_td(const BwdParams &p, void *workspace, size_t workspace_b
   DK_ALLOW_DYNAMIC_LDS((mfma_dkdv_kernel<T, D, PAD, SUB>), smem_dkdv);
   const int past = p.causal ? s.max_k_len - s.max_q_len : 0;
   const int tiles = (past + s.max_q_len - 1) / 64 - past / 64 + 1;
-  DK_REQUIRE(tiles <= 65535 && cdiv(s.max_k_len, 64) <= 65535 && p.csc.num_rows <= 65535, "sequence too long for one launch");
+  DK_REQUIRE(tiles <= 65535 && cdiv(s.max_k_len, 64) <= 65535 && p.csc.num_rows <= 65535 &&
+                 (!(p.csr.order || p.csr.pair_order) || p.csr.num_rows <= 65535),
+             "sequence too long for one launch");
   // dQ first: it also writes delta, which the dK/dV pass reads
   if constexpr (D <= 128) {  // two table rows per workgroup
-    const int pairs = (((past + s.max_q_len - 1) / 64) >> 1) - ((past / 64) >> 1) + 1;
+    int pairs = (((past + s.max_q_len - 1) / 64) >> 1) - ((past / 64) >> 1) + 1;
     DK_ALLOW_DYNAMIC_LDS((mfma_dq_pair_kernel<T, D, PAD, SUB>), smem_dq);
+    if (p.csr.pair_order) pairs = (p.csr.num_rows + 1) / 2;  // handed out in the table's order: all of them
     BwdParams pq = p;
     pq.csr.rot = head_rotation(p.csr, p.Hq, pairs);  // (uneven heads: dealt to the queues in rotation)
     DK_NOTE_KERNEL(pq.csr.rot ? "mfma_dq_pair_kernel, heads in rotation" : "mfma_dq_pair_kernel");
     hipLaunchKernelGGL((mfma_dq_pair_kernel<T, D, PAD, SUB>), dim3(p.Hq, pairs, s.batch), dim3(256), smem_dq, stream, pq, pairs);
   } else {
     DK_ALLOW_DYNAMIC_LDS((mfma_dq_kernel<T, D, PAD, SUB>), smem_dq);
+    const int rows = p.csr.order ? p.csr.num_rows : tiles;  // handed out in the table's order: all of them
     BwdParams pq = p;
-    pq.csr.rot = head_rotation(p.csr, p.Hq, tiles);
+    pq.csr.rot = head_rotation(p.csr, p.Hq, rows);
     DK_NOTE_KERNEL(pq.csr.rot ? "mfma_dq_kernel, heads in rotation" : "mfma_dq_kernel");
-    hipLaunchKernelGGL((mfma_dq_kernel<T, D, PAD, SUB>), dim3(p.Hq, tiles, s.batch), dim3(256), smem_dq, stream, pq, tiles);
+    hipLaunchKernelGGL((mfma_dq_kernel<T, D, PAD, SUB>), dim3(p.Hq, rows, s.batch), dim3(256), smem_dq, stream, pq, rows);
   }
   DK_HIP_CHECK(hipGetLastError());
   // With several q heads per kv head a workgroup per kv head walks all of them, and the longest

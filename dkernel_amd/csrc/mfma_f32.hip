@@ -108,7 +108,14 @@ __global__ __launch_bounds__(128) void fwd_kernel(const FwdParams p, int tiles_y
   __shared__ __align__(16) float sV[64 * kLd];
   SeqInfo sq;
   int tile;
-  const bool has_rows = resolve_tile(p.seqs, p.causal, 64, 1, tiles_y - 1 - (int)blockIdx.y, blockIdx.z, sq, tile);
+  bool has_rows;
+  if (p.csr.order && !p.seqs.packed) {  // the table's own order, longest rows first (the grid covers every row of it)
+    sq = load_seq(p.seqs, blockIdx.z, p.causal);
+    tile = p.csr.order[lut_head(p.csr, grid_head(p.csr), p.Hq, p.Hkv) * p.csr.order_sh + blockIdx.y] - sq.past / 64;
+    has_rows = tile >= 0 && tile < seq_row_blocks(sq, 64);
+  } else {
+    has_rows = resolve_tile(p.seqs, p.causal, 64, 1, tiles_y - 1 - (int)blockIdx.y, blockIdx.z, sq, tile);
+  }
   if (p.seqs.zero_outside)
     zero_rows_outside<float>(p.seqs, sq, blockIdx.y, tiles_y, p.o, p.lse, grid_head(p.csr), 1, p.D, p.vec_ok, threadIdx.x, 128);
   if (!has_rows) return;
@@ -221,11 +228,12 @@ __global__ __launch_bounds__(128) void dq_kernel(const BwdParams p, int tiles_y)
   __shared__ __align__(16) float sK[64 * kLd];
   __shared__ __align__(16) float sV[64 * kLd];
   const SeqInfo sq = load_seq(p.seqs, blockIdx.z, p.causal);
-  const int tile = tiles_y - 1 - (int)blockIdx.y;
-  if (tile >= seq_row_blocks(sq, 64)) return;
+  const int h = grid_head(p.csr), kvh = h / (p.Hq / p.Hkv);
+  int tile = tiles_y - 1 - (int)blockIdx.y;
+  if (p.csr.order) tile = p.csr.order[lut_head(p.csr, h, p.Hq, p.Hkv) * p.csr.order_sh + blockIdx.y] - sq.past / 64;
+  if (tile < 0 || tile >= seq_row_blocks(sq, 64)) return;
   const int rb = sq.past / 64 + tile;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int h = grid_head(p.csr), kvh = h / (p.Hq / p.Hkv);
   const int m = lane & 31, g = lane >> 5;
   const int row0 = rb * 64 + wave * 32;
   const int pos = row0 + m, qi = pos - sq.past;
@@ -385,6 +393,7 @@ int launch_mfma_f32_fwd(const FwdParams &p, hipStream_t stream) {
     const int past = p.causal ? s.max_k_len - s.max_q_len : 0;
     tiles = (past + s.max_q_len - 1) / 64 - past / 64 + 1;
   }
+  if (p.csr.order && !s.packed) tiles = p.csr.num_rows;  // handed out in the table's order: all of them
   DK_REQUIRE(tiles <= 65535, "too many q tiles for one launch (%d)", tiles);
   FwdParams pr = p;
   pr.csr.rot = head_rotation(p.csr, p.Hq, tiles);  // (uneven heads: dealt to the queues in rotation)
@@ -403,10 +412,12 @@ int launch_mfma_f32_bwd(const BwdParams &p, hipStream_t stream) {
   DK_NOTE_KERNEL("f32::delta_kernel");
   hipLaunchKernelGGL(f32::delta_kernel, dim3(cdiv(s.max_q_len, 16), p.Hq, s.batch), dim3(256), 0, stream, p);
   DK_HIP_CHECK(hipGetLastError());
+  DK_REQUIRE(!p.csr.order || p.csr.num_rows <= 65535, "sequence too long for one launch");
+  const int rows = p.csr.order ? p.csr.num_rows : tiles;  // handed out in the table's order: all of them
   BwdParams pq = p;
-  pq.csr.rot = head_rotation(p.csr, p.Hq, tiles);
+  pq.csr.rot = head_rotation(p.csr, p.Hq, rows);
   DK_NOTE_KERNEL(pq.csr.rot ? "f32::dq_kernel, heads in rotation" : "f32::dq_kernel");
-  hipLaunchKernelGGL(f32::dq_kernel, dim3(p.Hq, tiles, s.batch), dim3(128), 0, stream, pq, tiles);
+  hipLaunchKernelGGL(f32::dq_kernel, dim3(p.Hq, rows, s.batch), dim3(128), 0, stream, pq, rows);
   DK_HIP_CHECK(hipGetLastError());
   BwdParams po = p;  // the order only where heads do not line up with the hardware's 32 workgroup queues
   if (p.Hkv % 32 == 0) po.csc.order = nullptr;

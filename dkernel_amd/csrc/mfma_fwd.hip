@@ -77,8 +77,11 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
     } else {
       sq = load_seq(p.seqs, blockIdx.z, p.causal);
       first_rb = sq.past / 64, last_rb = (sq.past + sq.q_len - 1) / 64;
-      u = (first_rb >> 1) + tiles_y - 1 - (int)blockIdx.y;
-      if (sq.q_len <= 0 || u > (last_rb >> 1)) {  // no rows here: only the share of the padding rows, if asked
+      if (p.csr.pair_order)  // the table's own order, longest pairs first (the grid then covers every pair of it)
+        u = scalar_load(p.csr.pair_order + lut_head(p.csr, grid_head(p.csr), p.Hq, p.Hkv) * p.csr.order_sh + blockIdx.y);
+      else
+        u = (first_rb >> 1) + tiles_y - 1 - (int)blockIdx.y;
+      if (sq.q_len <= 0 || u > (last_rb >> 1) || u < (first_rb >> 1)) {  // no rows here: only the share of the padding rows, if asked
         if (p.seqs.zero_outside)
           zero_rows_outside<T>(p.seqs, sq, blockIdx.y, tiles_y, p.o, p.lse, grid_head(p.csr), 1, p.D, p.vec_ok, tid, NT);
         return;
@@ -87,8 +90,17 @@ __global__ __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(G == 1 
     rb = 2 * u + (wave >> 1);
     tile = rb - first_rb;  // outside [0, last_rb - first_rb]: this wave pair has no rows (row_ok false everywhere)
   } else {
-    const int ty = tiles_y - 1 - (int)blockIdx.y;  // longest rows first
-    if (!resolve_tile(p.seqs, p.causal, 64, 1, ty, blockIdx.z, sq, tile)) {
+    const int ty = tiles_y - 1 - (int)blockIdx.y;  // longest rows first (of a causal pattern)
+    bool has_rows;
+    if (p.csr.order && !p.seqs.packed) {  // the table's own order, longest rows first (the grid then covers every row of it)
+      sq = load_seq(p.seqs, blockIdx.z, p.causal);
+      tile = scalar_load(p.csr.order + lut_head(p.csr, grid_head(p.csr) * G, p.Hq, p.Hkv) * p.csr.order_sh + blockIdx.y) -
+             sq.past / 64;
+      has_rows = tile >= 0 && tile < seq_row_blocks(sq, 64);
+    } else {
+      has_rows = resolve_tile(p.seqs, p.causal, 64, 1, ty, blockIdx.z, sq, tile);
+    }
+    if (!has_rows) {
       if (p.seqs.zero_outside)  // (never with packed inputs, for which sq is not set here)
         zero_rows_outside<T>(p.seqs, sq, blockIdx.y, tiles_y, p.o, p.lse, grid_head(p.csr) * G, G, p.D, p.vec_ok, tid, NT);
       return;
@@ -531,6 +543,7 @@ static int launch_row_pairs(const FwdParams &p, hipStream_t stream) {
     const int past = p.causal ? s.max_k_len - s.max_q_len : 0;
     pairs = (((past + s.max_q_len - 1) / 64) >> 1) - ((past / 64) >> 1) + 1;
   }
+  if (p.csr.pair_order && !s.packed) pairs = (p.csr.num_rows + 1) / 2;  // handed out in the table's order: all of them
   DK_REQUIRE(pairs <= 65535, "too many q tiles for one launch (%d)", pairs);
   if (int rc = launch_item_offsets(p, true, stream)) return rc;
   const FwdParams pr = for_grid(p, p.Hq, pairs);
@@ -630,6 +643,7 @@ int launch_mfma_fwd(const FwdParams &p_in, int dtype, void *workspace, size_t wo
     const int past = p.causal ? s.max_k_len - s.max_q_len : 0;
     tiles = (past + s.max_q_len - 1) / 64 - past / 64 + 1;
   }
+  if (p.csr.order && !s.packed) tiles = p.csr.num_rows;  // handed out in the table's order: all of them
   DK_REQUIRE(tiles <= 65535, "too many q tiles for one launch (%d)", tiles);
   dim3 grid(1, tiles, s.packed ? 1 : s.batch);
   return dtype == DK_BF16 ? launch_t<bf16_t>(p, grid, tiles, stream) : launch_t<f16_t>(p, grid, tiles, stream);

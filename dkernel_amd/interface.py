@@ -54,6 +54,16 @@ def _uneven_heads(pattern: Tensor) -> bool:
     return bool(counts.max() * counts.numel() > 1.2 * counts.sum())
 
 
+def _unsorted_rows(pattern: Tensor) -> bool:
+    """True when some row of some head holds clearly more blocks (a quarter more, and at least
+    two) than every row after it: starting from the last row is then not longest first."""
+    lens = pattern.sum(2, dtype=torch.int64).cpu()
+    if lens.size(1) < 2:
+        return False
+    later = torch.flip(torch.cummax(torch.flip(lens, (1,)), dim=1).values, (1,))[:, 1:]  # longest later row
+    return bool((4 * lens[:, :-1] > 5 * later + 8).any())
+
+
 class SparseAttention(torch.nn.Module):
     """Block-sparse attention over a user-given block pattern.
 
@@ -134,6 +144,11 @@ class SparseAttention(torch.nn.Module):
         # prefill and backward kernels then deal the heads to the hardware's workgroup queues in
         # rotation, so that no part of the chip is left with the dense heads alone
         self.kwargs['uneven_heads'] = _uneven_heads(sparse_pattern)
+        # rows that are clearly longer than every row after them (global rows at the start of a
+        # non-causal pattern): the forward and dQ kernels, which otherwise start from the last row
+        # - the longest of a causal pattern -, then take the rows in the table's own order, longest
+        # first, instead of starting the long ones when the rest of the chip has run out of work
+        self.kwargs['unsorted_rows'] = _unsorted_rows(sparse_pattern)
 
         if not causal:
             # merged q tiles are a causal-only optimisation

@@ -105,10 +105,17 @@ def _lut(layout: Tuple[Tensor, Tensor, int, int], device, group: int = 1, max_ro
         order = None
         if longest_first:
             # rows of every head by descending length (stable: equal lengths stay in index order),
-            # computed on the device once per table: the dK/dV pass hands its columns out in this order
+            # computed on the device once per table: the dK/dV pass hands its columns out in this
+            # order, the forward and dQ kernels the rows of a pattern whose long rows are not its last
             ptr = layout[0] if layout[0].dim() == 2 else layout[0][None]
-            order = torch.argsort(ptr[:, 1:] - ptr[:, :-1], dim=1, descending=True, stable=True).to(torch.int32).contiguous()
+            lens = ptr[:, 1:] - ptr[:, :-1]
+            rows = lens.size(1)
+            # ... followed by the pairs of rows (2u, 2u + 1) by descending length of the pair
+            pair_lens = torch.nn.functional.pad(lens, (0, rows % 2)).view(lens.size(0), -1, 2).sum(2)
+            order = torch.cat([torch.argsort(x, dim=1, descending=True, stable=True) for x in (lens, pair_lens)],
+                              dim=1).to(torch.int32).contiguous()
             lut.row_order, lut.row_order_stride_h = order.data_ptr(), order.stride(0)
+            lut.pair_order = order.data_ptr() + 4 * rows
         hit = _LUT_CACHE[key] = (lut, layout[0], layout[1], order)
     return _lib.Lut.from_buffer_copy(hit[0])
 
@@ -198,7 +205,8 @@ def _forward(ctx, q: Tensor, k: Tensor, v: Tensor, sm_scale: float,
              split_qkv=None,
              lut_group: int = 1,
              lut_max_row: int = 0,
-             uneven_heads: bool = False) -> Tuple[Tensor, Optional[Tensor]]:
+             uneven_heads: bool = False,
+             unsorted_rows: bool = False) -> Tuple[Tensor, Optional[Tensor]]:
     """Unpadded 4-D forward (training, prefill, single-token decode).
     Reference: dkernel/ops/sparse_attn_fwd.py:383-567.  `d_splits` is accepted
     and ignored (a Triton shared-memory workaround)."""
@@ -225,7 +233,8 @@ def _forward(ctx, q: Tensor, k: Tensor, v: Tensor, sm_scale: float,
     args = _lib.FwdArgs()
     args.q, args.k, args.v, args.o = (_tensor4(x, hdim, seq_dim) for x in (q, k, v, o))
     args.lse = _rowvec(lse)
-    args.csr = _lut(layout_csr, q.device, lut_group, lut_max_row, uneven=uneven_heads)
+    args.csr = _lut(layout_csr, q.device, lut_group, lut_max_row, uneven=uneven_heads,
+                    longest_first=unsorted_rows and qlen > 1)
     args.seqs = _lib.Seqs(q.size(0), qlen, klen, 0, None, None, None, None)
     args.num_q_heads, args.num_kv_heads, args.head_dim = num_heads, num_kv_heads, q.size(-1)
     args.dtype, args.causal, args.impl = _DTYPES[q.dtype], int(bool(causal)), _impl
@@ -240,6 +249,7 @@ def _forward(ctx, q: Tensor, k: Tensor, v: Tensor, sm_scale: float,
     ctx.causal = causal
     ctx.lut_group = lut_group
     ctx.uneven_heads = uneven_heads
+    ctx.unsorted_rows = unsorted_rows
     return o, (lse if return_lse else None)
 
 
@@ -278,7 +288,8 @@ def _backward(ctx, do: Tensor, dlse: Optional[Tensor],
     if masked is not None and _matrix_core_applies(q, k, v, o, do, dq, dk, dv):
         layout_csr, layout_csc = masked[0], masked[1]
     uneven = getattr(ctx, "uneven_heads", False)
-    args.csr = _lut(layout_csr, q.device, ctx.lut_group, uneven=uneven)
+    args.csr = _lut(layout_csr, q.device, ctx.lut_group, uneven=uneven,
+                    longest_first=getattr(ctx, "unsorted_rows", False))
     args.csc = _lut(layout_csc, q.device, ctx.lut_group, longest_first=True, uneven=uneven)
     args.seqs = _lib.Seqs(B, Lq, k.size(seq_dim), 0, None, None, None, None)
     args.num_q_heads, args.num_kv_heads, args.head_dim = Hq, k.size(hdim), q.size(-1)
@@ -309,7 +320,8 @@ def padded_sparse_attn(q: Tensor, k: Tensor, v: Tensor, sm_scale: float,
                        return_lse: bool = False,
                        lut_group: int = 1,
                        lut_max_row: int = 0,
-                       uneven_heads: bool = False):
+                       uneven_heads: bool = False,
+                       unsorted_rows: bool = False):
     """4-D inputs with left paddings and / or explicit sequence lengths; q has
     either one token per sequence (decode) or the same padded length as k.
     Reference: dkernel/ops/sparse_attn_inference.py:10-147.  Padding rows of
@@ -361,7 +373,8 @@ def padded_sparse_attn(q: Tensor, k: Tensor, v: Tensor, sm_scale: float,
     args = _lib.FwdArgs()
     args.q, args.k, args.v, args.o = (_tensor4(x, hdim, seq_dim) for x in (q, k, v, out))
     args.lse = _rowvec(lse)
-    args.csr = _lut(sparse_layout, dev, lut_group, lut_max_row, uneven=uneven_heads and q_len > 1)
+    args.csr = _lut(sparse_layout, dev, lut_group, lut_max_row, uneven=uneven_heads and q_len > 1,
+                    longest_first=unsorted_rows and q_len > 1)
     args.seqs = _lib.Seqs(batches, q_len, k_len, 4 if clear_padding else 0, q_starts.data_ptr(), q_ends.data_ptr(),
                           k_starts.data_ptr(), k_ends.data_ptr())
     args.num_q_heads, args.num_kv_heads, args.head_dim = num_heads, num_kv_heads, head_size
@@ -587,14 +600,15 @@ class _sparse_attention(torch.autograd.Function):
                                          seqlens=seqlens, seq_dim=seq_dim, max_seqlen=max_seqlen,
                                          out=kwargs.get("out", None),
                                          causal=causal, return_lse=return_lse, lut_group=lut_group,
-                                         lut_max_row=lut_max_row, uneven_heads=kwargs.get("uneven_heads", False))
+                                         lut_max_row=lut_max_row, uneven_heads=kwargs.get("uneven_heads", False),
+                                         unsorted_rows=kwargs.get("unsorted_rows", False))
                 output, lse = res if return_lse else (res, None)
             else:
                 ctx.support_backward = True
                 ctx.message = ""
                 fwd_kwargs = {k_: v_ for k_, v_ in kwargs.items()
                               if k_ in ("inference", "out", "d_splits", "max_seqlen", "return_lse",
-                                        "causal", "split_qkv", "lut_group", "uneven_heads")}
+                                        "causal", "split_qkv", "lut_group", "uneven_heads", "unsorted_rows")}
                 fwd_kwargs["lut_max_row"] = lut_max_row
                 output, lse = _forward(ctx, q, k, v, sm_scale, layout_csr, seq_dim=seq_dim, **fwd_kwargs)
         return output, lse

@@ -126,7 +126,8 @@ typedef struct dk_lut {
   const int32_t *row_order; /* optional (NULL: ascending): row_order[h * row_order_stride_h + i] is
                                the table row that the i-th work item of head h takes, a
                                permutation of 0 .. num_rows-1 with the longest rows first.  Read
-                               by the dK/dV pass for its column table: workgroups are handed to
+                               by the dK/dV pass for its column table, and by the forward and dQ
+                               kernels for their row table (see pair_order): workgroups are handed to
                                the shader engines round-robin and in order, so long columns that
                                recur with a period (vertical strides) otherwise pile up on a few
                                of them while the rest wait behind a full queue. */
@@ -138,6 +139,16 @@ typedef struct dk_lut {
                            dense heads alone; with even heads (0) a fixed head per queue shares more
                            tiles through the caches.  Results do not depend on it. */
   int32_t reserved;     /* 0 */
+  const int32_t *pair_order; /* optional, with row_order on the row table of dk_fwd / dk_bwd (same head
+                                stride): pair_order[h * row_order_stride_h + i] is the pair u of table
+                                rows (2u, 2u + 1) that the i-th work item of head h takes in the kernels
+                                that work on two rows at a time, a permutation of
+                                0 .. (num_rows + 1) / 2 - 1 by descending length of the pair.  Without
+                                the two orders the forward and dQ kernels start from the last row, which
+                                is the longest of a causal pattern; a pattern whose long rows come
+                                first (global rows of a non-causal pattern) would start them last,
+                                with the rest of the chip idle while they finish.  Not read for packed
+                                inputs. */
 } dk_lut;
 
 /* Sequence geometry.  With all four pointers NULL every sequence has

@@ -34,9 +34,9 @@ def test_library_exports_every_declared_symbol():
 def test_struct_sizes_match_header():
     # natural alignment on x86-64: catches a field added on one side only
     assert ctypes.sizeof(_lib.Tensor) == 32 and ctypes.sizeof(_lib.RowVec) == 32
-    assert ctypes.sizeof(_lib.Lut) == 88 and ctypes.sizeof(_lib.Seqs) == 48
-    assert ctypes.sizeof(_lib.FwdArgs) == 4 * 32 + 32 + 88 + 48 + 7 * 4 + 4 + 3 * 8
-    assert ctypes.sizeof(_lib.BwdArgs) == 8 * 32 + 2 * 32 + 8 + 2 * 88 + 48 + 7 * 4 + 4 + 3 * 8
+    assert ctypes.sizeof(_lib.Lut) == 96 and ctypes.sizeof(_lib.Seqs) == 48
+    assert ctypes.sizeof(_lib.FwdArgs) == 4 * 32 + 32 + 96 + 48 + 7 * 4 + 4 + 3 * 8
+    assert ctypes.sizeof(_lib.BwdArgs) == 8 * 32 + 2 * 32 + 8 + 2 * 96 + 48 + 7 * 4 + 4 + 3 * 8
     assert ctypes.sizeof(_lib.CombineArgs) == 6 * 4 + 2 * 32 + 4 * 8 * 32 + 8
 
 
@@ -424,17 +424,36 @@ def test_longest_first_order_of_a_table():
     _, mask, _ = get_sparse_attn_mask(4, 1024, block_size=64, local_blocks=2, vert_stride=4, dtype=torch.uint8)
     ccol, row = dense_to_ccol_row(mask.to(torch.uint8))
     lut = ops._lut((ccol, row, 64, 64), ccol.device, longest_first=True)
-    assert lut.row_order and lut.row_order_stride_h == 16
-    order = np.ctypeslib.as_array(ctypes.cast(lut.row_order, ctypes.POINTER(ctypes.c_int32)), shape=(ccol.size(0), 16))
+    # 16 rows, followed by the 8 pairs of rows (2u, 2u + 1) in the order of the pairs' lengths
+    assert lut.row_order and lut.row_order_stride_h == 24 and lut.pair_order == lut.row_order + 4 * 16
+    both = np.ctypeslib.as_array(ctypes.cast(lut.row_order, ctypes.POINTER(ctypes.c_int32)), shape=(ccol.size(0), 24))
     lens = (ccol[:, 1:] - ccol[:, :-1]).numpy()
-    for h in range(ccol.size(0)):
-        assert sorted(order[h]) == list(range(16))
-        got = lens[h][order[h]]
-        assert (np.diff(got) <= 0).all()
-        for a, b in zip(order[h][:-1], order[h][1:]):
-            assert lens[h][a] > lens[h][b] or a < b
+    for order, lens_of in ((both[:, :16], lens), (both[:, 16:], lens[:, 0::2] + lens[:, 1::2])):
+        n = order.shape[1]
+        for h in range(ccol.size(0)):
+            assert sorted(order[h]) == list(range(n))
+            got = lens_of[h][order[h]]
+            assert (np.diff(got) <= 0).all()
+            for a, b in zip(order[h][:-1], order[h][1:]):
+                assert lens_of[h][a] > lens_of[h][b] or a < b
     plain = ops._lut((ccol, row, 64, 64), ccol.device)
-    assert not plain.row_order
+    assert not plain.row_order and not plain.pair_order
+
+
+def test_which_patterns_start_their_long_rows_first():
+    from dkernel_amd.interface import _unsorted_rows
+    for kw in (dict(), dict(homo_head=True), dict(head_sliding_offset=1), dict(num_dense_heads=2), dict(causal=False)):
+        for local, vert in ((2, 4), (8, 8), (1, 3), (16, 1)):
+            mask = torch.from_numpy(OL.block_mask(8, 4096, 64, local, vert, **kw).astype("uint8"))
+            assert not _unsorted_rows(mask), (kw, local, vert)
+    i = torch.arange(64)
+    window = (i[:, None] - i[None, :]).abs() <= 3
+    with_global = window.clone()
+    with_global[:2, :] = True
+    with_global[:, :2] = True
+    assert not _unsorted_rows(window[None].to(torch.uint8))
+    assert _unsorted_rows(with_global[None].to(torch.uint8))           # global rows first, the longest by far
+    assert not _unsorted_rows((with_global & (i[:, None] >= i[None, :]))[None].to(torch.uint8))  # causal: rows only grow
 
 
 def test_which_patterns_count_as_uneven():

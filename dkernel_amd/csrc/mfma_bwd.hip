@@ -716,8 +716,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 
   const int kvh = head_split ? __builtin_amdgcn_readfirstlane(out_head / ratio) : out_head;
   const int gq_first = head_split ? out_head - kvh * ratio : 0;
   const int gq_end = head_split ? gq_first + 1 : ratio;
-  // Columns are handed out longest first when the table says in which order: the hardware deals workgroups to its shader engines round-robin
-  // and in order, so long columns that recur with a period pile up on a few engines otherwise.
+  // Columns are handed out longest first when the table says in which order: the hardware deals
+  // workgroups to its shader engines round-robin and in order, so long columns that recur with a
+  // period pile up on a few engines otherwise.
   int cb = blockIdx.y;
   if (p.csc.order)  // (the grid then covers every column of the table)
     cb = scalar_load(p.csc.order + lut_head(p.csc, kvh * ratio + gq_first, p.Hq, p.Hkv) * p.csc.order_sh + blockIdx.y);

@@ -290,7 +290,9 @@ def test_random_user_pattern_matches_generic_kernels_and_oracle(seed):
         if name == "LSE":
             assert_close(f"{name} auto vs generic", a, b, atol=LSE_TOL, rtol=0)
         else:
-            assert_close(f"{name} auto vs generic", a, b, **TOL)
+            # two 16-bit results, each held to TOL against the oracle below: between themselves
+            # their errors add (1 element in 44 416 of one seed in 5 800 differed by 0.0225)
+            assert_close(f"{name} auto vs generic", a, b, atol=1.5 * TOL["atol"], rtol=1.5 * TOL["rtol"])
     bm = expand_heads(pat.numpy(), H)
     qo, ko, vo = (x.float().requires_grad_(True) for x in (q, k, v))
     ro, rl = oracle_fwd(qo, ko, vo, bm, bs, sm, seq_dim=1, causal=causal)
